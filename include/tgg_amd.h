@@ -1,0 +1,105 @@
+/* C ABI of the MI355X (gfx950) grouped-GEMM library, libtgg_amd.so.
+ *
+ * Every entry point takes raw device pointers, plain sizes and the HIP stream to
+ * enqueue on (a hipStream_t passed as void*; NULL = the default stream).  Calls
+ * are asynchronous: they validate their arguments on the host, launch, and
+ * return.  Return value 0 = enqueued; 1 = rejected argument; 2 = HIP runtime
+ * error.  tgg_last_error() gives the message of the calling thread's last
+ * failure.  No entry point allocates, frees or synchronises.
+ *
+ * Each declaration cites the reference interface it stands in for
+ * (paths relative to the DeepLink-org/Triton_Grouped_GEMM tree).
+ */
+#ifndef TGG_AMD_H_
+#define TGG_AMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type codes */
+#define TGG_BF16 0
+#define TGG_F16 1
+#define TGG_E4M3 2 /* OCP float8_e4m3fn */
+#define TGG_E5M2 3 /* OCP float8_e5m2 */
+
+#define TGG_MAX_GROUPS 1024
+
+/* C[r,:] = A[r,:] . B[g(r)]^T (trans_b=1, B is [G,N,K]) or A[r,:] . B[g(r)] (trans_b=0, B is [G,K,N]);
+ * rows of group g are the sizes[g] rows after those of groups < g; fp32 accumulate, output in `dtype`.
+ * Replaces m_grouped_gemm / _m_grouped_gemm_launch + _build_m_grouped_metadata
+ * (gemm/BF16/m_grouped_gemm_TMA.py:297-447; SM80 twin gemm/BF16/m_grouped_gemm.py:220-292). */
+int tgg_m_grouped_gemm(const void* A, const void* B, void* C, const void* sizes, int sizes_i64, int G, int64_t M,
+                       int N, int K, int trans_b, int dtype, int num_cu, void* stream);
+
+/* Same contraction with A/C physically padded: group g starts at sum_{h<g} round_up(sizes[h], align).
+ * Replaces deep_gemm.m_grouped_bf16_gemm_nt_contiguous as called from m_grouped_bf16_nt_contiguous
+ * (gemm/deep_gemm_ops.py:24-57).  Pad rows of C are not written. */
+int tgg_m_grouped_gemm_padded(const void* A, const void* B, void* C, const void* sizes, int sizes_i64, int G,
+                              int64_t M, int N, int K, int align, int dtype, int num_cu, void* stream);
+
+/* For each g and r < masked_m[g]: C[g*m_stride + r,:] = A[g*m_stride + r,:] . B[g]^T (trans_b=1, B [G,N,K]) or
+ * . B[g] (trans_b=0, B [G,K,N]); other rows untouched.  Replaces m_grouped_gemm_masked
+ * (gemm/BF16/m_grouped_gemm_masked_TMA.py:164-250); m_stride is its expected_m. */
+int tgg_m_grouped_gemm_masked(const void* A, const void* B, void* C, const void* masked_m, int masked_i64, int G,
+                              int64_t m_stride, int64_t M, int N, int K, int trans_b, int dtype, int num_cu,
+                              void* stream);
+
+/* C[g] = A[start[g]:end[g], :]^T . B[start[g]:end[g], :], A [Ktot,Mdim], B [Ktot,N], C [G,Mdim,N];
+ * empty segments give zeros.  Replaces k_grouped_gemm (gemm/BF16/k_grouped_gemm_TMA.py:217-294;
+ * SM80 twin gemm/BF16/k_grouped_gemm.py:142-216). */
+int tgg_k_grouped_gemm(const void* A, const void* B, void* C, const int32_t* start, const int32_t* end, int G,
+                       int Mdim, int N, int64_t Ktot, int dtype, int num_cu, void* stream);
+
+/* C = (Aq . Bq[g]^T) * a_scale[r] * b_scale[g*N+n].  Replaces gmm_fp8_act_per_channel_w_per_expert
+ * (gemm/FP8/m_grouped_gemm_channel_expert.py:139-198). */
+int tgg_m_grouped_gemm_fp8_channel(const void* Aq, const float* a_scale, const void* Bq, const float* b_scale,
+                                   void* C, const void* sizes, int sizes_i64, int G, int64_t M, int N, int K,
+                                   int fmt_a, int fmt_b, int out_dtype, int num_cu, void* stream);
+
+/* out[g] = (x[:,seg_g] . y[:,seg_g]^T) * xs[g*M+m] * ys[g*N+n], x [M,Ktot], y [N,Ktot], segments =
+ * prefix sums of tokens[g]; bf16 output [G,M,N].  Replaces matmul
+ * (gemm/FP8/k_grouped_gemm_channel_expert.py:143-181). */
+int tgg_k_grouped_gemm_fp8_channel(const void* x, const float* xs, const void* y, const float* ys, void* out,
+                                   const int32_t* tokens, int G, int M, int N, int64_t Ktot, int fmt_a, int fmt_b,
+                                   int num_cu, void* stream);
+
+/* out[r,n] = sum_kb (sum_{k in kb} Aq[r,k] Bq[g,n,k]) * sa[r,kb] * sb[g,n/128,kb]; e4m3fn codes, A physically
+ * padded per group to `align` rows, sa [M,ceil(K/128)], sb [G,ceil(N/128),ceil(K/128)], bf16 output.
+ * Replaces deep_gemm.m_grouped_fp8_gemm_nt_contiguous as called from m_grouped_fp8_nt_contiguous
+ * (gemm/deep_gemm_ops.py:60-100). */
+int tgg_m_grouped_gemm_fp8_block(const void* Aq, const float* sa, const void* Bq, const float* sb, void* C,
+                                 const void* sizes, int sizes_i64, int G, int64_t M, int N, int K, int align,
+                                 int num_cu, void* stream);
+
+/* bf16 x [M,N] -> codes [N,M_expand] (transposed, each group padded to 128 columns, zero tail) and
+ * scales [N/128, M_expand/128].  Replaces trans_per_block_quant_expand_128x
+ * (quant/trans_per_block_quant_expand_128x.py:135-208). */
+int tgg_trans_per_block_quant_expand_128x(const void* x, void* codes, float* scales, const void* sizes,
+                                          int sizes_i64, int G, int64_t M, int N, int64_t M_expand, int fmt,
+                                          void* stream);
+
+/* bf16 x [M,K] -> codes [M,K], scales [M,K/128]; 1x128 recipe.  Replaces per_token_cast_to_fp8
+ * (gemm/FP8/m_grouped_gemm_channel_expert.py:217-222). */
+int tgg_per_token_cast_to_fp8(const void* x, void* codes, float* scales, int64_t M, int K, int fmt, void* stream);
+
+/* bf16 x [batch,R,C] -> codes (same shape), scales [batch,ceil(R/128),ceil(C/128)]; 128x128 recipe.
+ * Replaces per_block_cast_to_fp8 (gemm/FP8/m_grouped_gemm_channel_expert.py:237-245). */
+int tgg_per_block_cast_to_fp8(const void* x, void* codes, float* scales, int batch, int R, int C, int fmt,
+                              void* stream);
+
+/* Element-wise fp32 -> fp8 code with the conversion the quantizers use (test hook for the
+ * `.to(torch.float8_*)` casts of the recipes above). */
+int tgg_cvt_f32_to_fp8(const float* in, void* out, int64_t n, int fmt, void* stream);
+
+/* Library controls: "force_generic" (0/1) routes every GEMM through the shape-agnostic kernel. */
+int tgg_set_option(const char* key, int value);
+const char* tgg_last_error(void);
+int tgg_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TGG_AMD_H_ */

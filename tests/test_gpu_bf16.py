@@ -1,0 +1,217 @@
+"""GPU parity: BF16/FP16 M-grouped, masked and K-grouped GEMM through the C ABI vs the CPU oracle."""
+import pytest
+import torch
+
+from oracle import gemm_ref
+from tests._util import check_16bit_gemm
+from triton_grouped_gemm_amd import _native, workloads
+from triton_grouped_gemm_amd.gemm.BF16.k_grouped_gemm_TMA import k_grouped_gemm
+from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm_masked_TMA import m_grouped_gemm_masked
+from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm_TMA import m_grouped_gemm
+from triton_grouped_gemm_amd.gemm.deep_gemm_ops import m_grouped_bf16_nt_contiguous
+
+pytestmark = pytest.mark.gpu
+
+
+def _randn(shape, scale, seed, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def _ints(shape, seed, dtype=torch.bfloat16, lo=-1, hi=1):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(lo, hi + 1, shape, generator=g).to(dtype)
+
+
+@pytest.fixture(params=[0, 1], ids=["tuned", "generic"])
+def variant(request, dev):
+    _native.set_option("force_generic", request.param)
+    yield request.param
+    _native.set_option("force_generic", 0)
+
+
+def test_config1_tiny_reference_case(dev, variant):
+    """BASELINE config 1: G=4, rows [64,128,32,96], K=256, N=512, seed 0, trans_b=True."""
+    torch.manual_seed(0)
+    sizes = torch.tensor([64, 128, 32, 96], dtype=torch.int32)
+    a = (torch.randn(320, 256) / 16).to(torch.bfloat16)
+    b = (torch.randn(4, 512, 256) / 16).to(torch.bfloat16)
+    out = m_grouped_gemm(a.to(dev), b.to(dev), sizes.to(dev), True)
+    rd = check_16bit_gemm(out, gemm_ref.gmm(a, b, sizes, True), gemm_ref.gmm_fp32(a, b, sizes, True), "config1")
+    print(f"config1 max-norm rdiff vs bf16 torch reference: {rd:.3e}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("trans_b", [True, False])
+@pytest.mark.parametrize("sizes,N,K", [
+    ([64, 128, 32, 96], 512, 256),
+    ([1, 0, 127, 129, 256, 3, 0, 300], 136, 72),
+    ([0, 0, 5], 8, 8),
+    ([200] * 16, 264, 64),
+])
+def test_m_grouped_exact_on_integer_inputs(dev, variant, dtype, trans_b, sizes, N, K):
+    """Entries in {-1,0,1}: every partial sum is an integer <= K <= 256, exactly representable, so the
+    result must equal the oracle bit for bit (catches any indexing / scheduling / masking slip)."""
+    M = sum(sizes)
+    a = _ints((M, K), 1, dtype)
+    b = _ints((len(sizes), N, K) if trans_b else (len(sizes), K, N), 2, dtype)
+    s = torch.tensor(sizes, dtype=torch.int32)
+    out = m_grouped_gemm(a.to(dev), b.to(dev), s.to(dev), trans_b)
+    ref = gemm_ref.gmm_fp32(a, b, sizes, trans_b).to(dtype)
+    assert torch.equal(out.cpu(), ref)
+
+
+@pytest.mark.parametrize("trans_b", [True, False])
+@pytest.mark.parametrize("sizes_dtype", [torch.int32, torch.int64])
+def test_m_grouped_random_ragged(dev, variant, trans_b, sizes_dtype):
+    sizes = [130, 0, 1, 255, 384, 77, 128, 49]
+    M, N, K = sum(sizes), 384, 320
+    a = _randn((M, K), K ** -0.5, 3)
+    b = _randn((8, N, K) if trans_b else (8, K, N), 1.0, 4)
+    s = torch.tensor(sizes, dtype=sizes_dtype)
+    out = m_grouped_gemm(a.to(dev), b.to(dev), s.to(dev), trans_b)
+    check_16bit_gemm(out, gemm_ref.gmm(a, b, sizes, trans_b), gemm_ref.gmm_fp32(a, b, sizes, trans_b), "ragged")
+
+
+def test_m_grouped_rows_past_sum_untouched_and_neighbours_do_not_leak(dev, variant):
+    """sum(sizes) < M: trailing rows keep their previous contents; a NaN row next to a group
+    boundary must not contaminate the neighbouring group's rows."""
+    from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm import _m_grouped_gemm_launch
+    sizes = [100, 60]
+    M, N, K = 192, 128, 64
+    a = _randn((M, K), 0.125, 5)
+    a[160:] = float("nan")
+    b = _randn((2, N, K), 1.0, 6)
+    c = torch.full((M, N), 7.0, dtype=torch.bfloat16, device=dev)
+    _m_grouped_gemm_launch(a.to(dev), b.to(dev), c, torch.tensor(sizes, dtype=torch.int32, device=dev), True)
+    c = c.cpu()
+    assert torch.equal(c[160:], torch.full((32, N), 7.0, dtype=torch.bfloat16))
+    check_16bit_gemm(c[:160], gemm_ref.gmm(a[:160], b, sizes, True), gemm_ref.gmm_fp32(a[:160], b, sizes, True), "leak")
+    # group-to-expert mapping: swapping the experts changes the answer accordingly
+    a2 = a.clone()
+    a2[100] = float("nan")  # first row of group 1
+    c2 = m_grouped_gemm(a2.to(dev), b.to(dev), torch.tensor(sizes, dtype=torch.int32, device=dev), True).cpu()
+    assert torch.isnan(c2[100].float()).all() and torch.isfinite(c2[:100].float()).all()
+    assert torch.isfinite(c2[101:160].float()).all()
+
+
+def test_m_grouped_runs_on_callers_stream_and_with_cpu_sizes(dev):
+    sizes = [256, 128]
+    a = _randn((384, 128), 0.1, 7)
+    b = _randn((2, 256, 128), 1.0, 8)
+    st = torch.cuda.Stream(device=dev)
+    with torch.cuda.stream(st):
+        out = m_grouped_gemm(a.to(dev), b.to(dev), torch.tensor(sizes, dtype=torch.int32), True, numSM=16)
+    st.synchronize()
+    check_16bit_gemm(out, gemm_ref.gmm(a, b, sizes, True), gemm_ref.gmm_fp32(a, b, sizes, True), "stream")
+
+
+def test_contiguous_padded_bf16(dev, variant):
+    sizes = [100, 0, 128, 300]
+    padded = [128, 0, 128, 384]
+    Mp, N, K = sum(padded), 256, 128
+    a = _randn((Mp, K), K ** -0.5, 9)
+    b = _randn((4, N, K), 1.0, 10)
+    out = torch.full((Mp, N), 3.0, dtype=torch.bfloat16, device=dev)
+    m_grouped_bf16_nt_contiguous(a.to(dev), b.to(dev), torch.tensor(sizes, dtype=torch.int32, device=dev), out=out)
+    out = out.cpu()
+    start = 0
+    for g, (s, p) in enumerate(zip(sizes, padded)):
+        if s:
+            check_16bit_gemm(out[start:start + s], a[start:start + s] @ b[g].t(),
+                             a[start:start + s].float() @ b[g].float().t(), f"padded g{g}")
+        assert torch.equal(out[start + s:start + p], torch.full((p - s, N), 3.0, dtype=torch.bfloat16))
+        start += p
+
+
+@pytest.mark.parametrize("trans_b", [True, False])
+def test_masked_small(dev, variant, trans_b):
+    G, m_max, N, K = 6, 256, 264, 192
+    masked = [0, 256, 1, 129, 77, 200]
+    lhs = _randn((G * m_max, K), K ** -0.5, 11)
+    for g, mm in enumerate(masked):  # rows beyond masked_m are garbage
+        lhs[g * m_max + mm:(g + 1) * m_max] = float("nan")
+    rhs = _randn((G, N, K), 1.0, 12)
+    rhs_in = rhs if trans_b else rhs.transpose(1, 2).contiguous()
+    out = torch.full((G * m_max, N), -5.0, dtype=torch.bfloat16, device=dev)
+    ret = m_grouped_gemm_masked(lhs.to(dev), rhs_in.to(dev), out, torch.tensor(masked, dtype=torch.int32, device=dev),
+                                m_max, trans_b)
+    assert ret is None
+    out = out.cpu()
+    refs = gemm_ref.masked_gmm(lhs, rhs, masked, m_max)
+    refs32 = gemm_ref.masked_gmm(lhs, rhs, masked, m_max, fp32=True)
+    for g, mm in enumerate(masked):
+        blk = out[g * m_max:(g + 1) * m_max]
+        if mm:
+            check_16bit_gemm(blk[:mm], refs[g], refs32[g], f"masked g{g}")
+        assert torch.equal(blk[mm:], torch.full((m_max - mm, N), -5.0, dtype=torch.bfloat16))
+
+
+def test_masked_full_mask_reduces_to_bmm_exact(dev, variant):
+    G, m_max, N, K = 4, 128, 128, 64
+    lhs = _ints((G * m_max, K), 13)
+    rhs = _ints((G, N, K), 14)
+    out = torch.empty((G * m_max, N), dtype=torch.bfloat16, device=dev)
+    m_grouped_gemm_masked(lhs.to(dev), rhs.to(dev), out, torch.full((G,), m_max, dtype=torch.int64, device=dev), m_max)
+    ref = torch.bmm(lhs.float().view(G, m_max, K), rhs.float().transpose(1, 2)).to(torch.bfloat16)
+    assert torch.equal(out.cpu().view(G, m_max, N), ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("sizes,Mdim,N", [
+    ([128, 256, 0, 64], 256, 128),
+    ([1, 33, 0, 130, 7], 136, 72),
+    ([512], 128, 384),
+])
+def test_k_grouped_exact_on_integer_inputs(dev, variant, dtype, sizes, Mdim, N):
+    """Entries in {-1,0,1} and every group <= 512 tokens... sums stay below 256 in magnitude with
+    overwhelming probability; verified on the oracle side before comparing bit for bit."""
+    Kt = sum(sizes)
+    a = _ints((Kt, Mdim), 15, dtype)
+    b = _ints((Kt, N), 16, dtype)
+    ref32 = gemm_ref.gmm_dw(a, b, sizes, fp32=True)
+    assert ref32.abs().max() <= 256
+    s = torch.tensor(sizes, dtype=torch.int32, device=dev)
+    out = k_grouped_gemm(a.to(dev), b.to(dev), s)
+    assert out.shape == (len(sizes), Mdim, N)
+    assert torch.equal(out.cpu(), ref32.to(dtype))
+
+
+def test_k_grouped_random_with_explicit_bounds(dev, variant):
+    sizes = [300, 0, 1000, 77, 128]
+    Kt, Mdim, N = sum(sizes), 384, 264
+    a = _randn((Kt, Mdim), 1.0, 17)
+    b = _randn((Kt, N), 1.0, 18)
+    s = torch.tensor(sizes, dtype=torch.int64, device=dev)
+    end = s.cumsum(0)
+    out = k_grouped_gemm(a.to(dev), b.to(dev), s, group_start=end - s, group_end=end)
+    ref, ref32 = gemm_ref.gmm_dw(a, b, sizes), gemm_ref.gmm_dw(a, b, sizes, fp32=True)
+    assert torch.count_nonzero(out[1]) == 0  # empty group -> zeros
+    for g in (0, 2, 3, 4):
+        check_16bit_gemm(out[g], ref[g], ref32[g], f"kgrouped g{g}")
+
+
+def test_k_grouped_single_group_is_plain_transposed_matmul(dev, variant):
+    a = _randn((640, 128), 1.0, 19)
+    b = _randn((640, 256), 1.0, 20)
+    out = k_grouped_gemm(a.to(dev), b.to(dev), torch.tensor([640], dtype=torch.int32, device=dev))
+    check_16bit_gemm(out[0], a.t() @ b, a.float().t() @ b.float(), "kgrouped G=1")
+
+
+def test_medium_dirichlet_config_shape(dev, variant):
+    """Config-2 style draw at 1/16 scale: G=128 experts, 40960 rows in 128-row blocks, gate-up shape."""
+    G, M, N, K = 128, 40960, 1536, 2048
+    sizes = workloads.dirichlet_multinomial_sizes(G, M, 128, seed=21)
+    assert int(sizes.sum()) == M
+    a = workloads.randn_bf16((M, K), K ** -0.5, 22)
+    b = workloads.randn_bf16((G, N, K), K ** -0.5, 23)
+    out = m_grouped_gemm(a.to(dev), b.to(dev), sizes.to(dev), True)
+    # oracle on a sample of groups (CPU time) -- the largest, the smallest non-empty, and two more
+    order = torch.argsort(sizes)
+    nz = [int(i) for i in order if sizes[i] > 0]
+    starts = (sizes.cumsum(0) - sizes).tolist()
+    for g in {nz[0], nz[-1], nz[len(nz) // 2], nz[len(nz) // 3]}:
+        s0, n = starts[g], int(sizes[g])
+        n = min(n, 512)
+        ag = a[s0:s0 + n]
+        check_16bit_gemm(out[s0:s0 + n], ag @ b[g].t(), ag.float() @ b[g].float().t(), f"medium g{g}")

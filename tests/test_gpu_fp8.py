@@ -1,0 +1,172 @@
+"""GPU parity: FP8 grouped GEMMs (per-channel x per-expert scales, block scales) through the C ABI.
+
+Tolerance: rdiff = max|out-ref| / max(max|out|, max|ref|) <= 2e-2 against the fp32 matmul of the
+dequantised operands (the stated FP8 target); integer-valued cases must be exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm_ref, quant_ref
+from tests._util import to_np_f32
+from triton_grouped_gemm_amd import _native
+from triton_grouped_gemm_amd.gemm.deep_gemm_ops import m_grouped_fp8_nt_contiguous
+from triton_grouped_gemm_amd.gemm.FP8.k_grouped_gemm_channel_expert import matmul
+from triton_grouped_gemm_amd.gemm.FP8.m_grouped_gemm_channel_expert import gmm_fp8_act_per_channel_w_per_expert
+
+pytestmark = pytest.mark.gpu
+FP8_RDIFF = 2e-2
+TORCH_FP8 = {"e4m3fn": torch.float8_e4m3fn, "e5m2": torch.float8_e5m2}
+
+
+def _randn(shape, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(torch.bfloat16)
+
+
+def _codes_to_torch(codes: np.ndarray, fmt: str) -> torch.Tensor:
+    return torch.from_numpy(codes.copy()).view(TORCH_FP8[fmt])
+
+
+@pytest.fixture(params=[0, 1], ids=["tuned", "generic"])
+def variant(request, dev):
+    _native.set_option("force_generic", request.param)
+    yield request.param
+    _native.set_option("force_generic", 0)
+
+
+@pytest.mark.parametrize("fmt_a,fmt_b", [("e4m3fn", "e4m3fn"), ("e5m2", "e4m3fn"), ("e4m3fn", "e5m2"), ("e5m2", "e5m2")])
+@pytest.mark.parametrize("dtype_out", [torch.bfloat16, torch.float16])
+def test_fp8_channel_m_grouped(dev, variant, fmt_a, fmt_b, dtype_out):
+    """The reference's own example layout (gemm/FP8/m_grouped_gemm_channel_expert.py:293-315) at small size:
+    per-token activation scale, per-expert weight scale expanded to [G*N]."""
+    sizes = [125, 0, 259, 128, 3]
+    M, N, K = sum(sizes), 264, 256
+    x = to_np_f32(_randn((M, K), 30))
+    w = to_np_f32(_randn((len(sizes), N, K), 31))
+    xq, xs = quant_ref.per_row_cast_to_fp8(x, fmt_a)
+    wq, ws = quant_ref.per_expert_cast_to_fp8(w, fmt_b)
+    ws_exp = np.repeat(ws, N, axis=1).reshape(-1)  # .view(-1,1).repeat(1,N)
+    out = gmm_fp8_act_per_channel_w_per_expert(
+        _codes_to_torch(xq, fmt_a).to(dev), torch.from_numpy(xs).to(dev), _codes_to_torch(wq, fmt_b).to(dev),
+        torch.from_numpy(ws_exp).to(dev), torch.tensor(sizes, dtype=torch.int32, device=dev), dtype_out)
+    assert out.dtype == dtype_out and out.shape == (M, N)
+    ref = gemm_ref.fp8_channel_reference(torch.from_numpy(quant_ref.dequant(xq, fmt_a)), torch.from_numpy(xs),
+                                         torch.from_numpy(quant_ref.dequant(wq, fmt_b)), torch.from_numpy(ws_exp), sizes)
+    rd = gemm_ref.rdiff(out.cpu().float(), ref)
+    assert rd <= FP8_RDIFF, rd
+    # fp32 accumulation of exactly representable products: only the 16-bit output rounding remains
+    assert rd <= (2.0 ** -7 if dtype_out == torch.bfloat16 else 2.0 ** -10)
+
+
+def test_fp8_channel_exact_on_integer_codes(dev, variant):
+    sizes = [64, 1, 191]
+    M, N, K = 256, 128, 128
+    g = torch.Generator().manual_seed(32)
+    xa = torch.randint(-2, 3, (M, K), generator=g).float()
+    wb = torch.randint(-2, 3, (3, N, K), generator=g).float()
+    sa = torch.tensor([0.5, 1.0, 2.0, 4.0])[torch.randint(0, 4, (M,), generator=g)]
+    sb = torch.tensor([0.25, 1.0])[torch.randint(0, 2, (3 * N,), generator=g)]
+    out = gmm_fp8_act_per_channel_w_per_expert(
+        xa.to(torch.float8_e4m3fn).to(dev), sa.view(-1, 1).to(dev), wb.to(torch.float8_e4m3fn).to(dev), sb.to(dev),
+        torch.tensor(sizes, dtype=torch.int64, device=dev), torch.bfloat16)
+    ref = gemm_ref.fp8_channel_reference(xa, sa, wb, sb, sizes)
+    assert ref.abs().max() <= 2048 and torch.equal(ref, ref.to(torch.bfloat16).float())
+    assert torch.equal(out.cpu().float(), ref)
+
+
+@pytest.mark.parametrize("dtype_a,dtype_b", [(1, 1), (2, 1)])
+def test_fp8_k_grouped_channel(dev, variant, dtype_a, dtype_b):
+    """Layout of the reference's generator (gemm/FP8/k_grouped_gemm_channel_expert.py:238-268): tokens of
+    every expert zero-padded to 128, scales [rows, G] stored expert-major."""
+    fa, fb = ("e4m3fn" if dtype_a == 1 else "e5m2"), ("e4m3fn" if dtype_b == 1 else "e5m2")
+    tokens = [125, 300, 0, 128]
+    padded = [(t + 127) // 128 * 128 for t in tokens]
+    M, N, G = 136, 264, len(tokens)
+    xq_l, xs_l, yq_l, ys_l = [], [], [], []
+    for i, (t, p) in enumerate(zip(tokens, padded)):
+        x = np.zeros((M, p), np.float32)
+        y = np.zeros((N, p), np.float32)
+        x[:, :t] = to_np_f32(_randn((M, t), 40 + i))
+        y[:, :t] = to_np_f32(_randn((N, t), 50 + i))
+        if p == 0:
+            xq, xs = np.zeros((M, 0), np.uint8), np.full((M, 1), 1e-4 / 448, np.float32)
+            yq, ys = np.zeros((N, 0), np.uint8), np.full((N, 1), 1e-4 / 448, np.float32)
+        else:
+            xq, xs = quant_ref.per_row_cast_to_fp8(x, fa)
+            yq, ys = quant_ref.per_row_cast_to_fp8(y, fb)
+        xq_l.append(xq); xs_l.append(xs); yq_l.append(yq); ys_l.append(ys)
+    xq, yq = np.concatenate(xq_l, 1), np.concatenate(yq_l, 1)
+    xs, ys = np.concatenate(xs_l, 1), np.concatenate(ys_l, 1)
+    Kt = sum(padded)
+    xs_t = torch.from_numpy(xs).t().contiguous().t().to(dev)  # [M, G] with strides (1, M), as the reference builds it
+    ys_t = torch.from_numpy(ys).to(dev)                        # plain contiguous [N, G]: logical indexing must still hold
+    out = matmul(_codes_to_torch(xq, fa).to(dev), xs_t, _codes_to_torch(yq, fb).to(dev), ys_t,
+                 torch.tensor(padded, dtype=torch.int32, device=dev), M, N, Kt, G, dtype_a, dtype_b)
+    assert out.shape == (G, M, N) and out.dtype == torch.bfloat16
+    ref = gemm_ref.fp8_k_grouped_channel_reference(torch.from_numpy(quant_ref.dequant(xq, fa)), torch.from_numpy(xs),
+                                                   torch.from_numpy(quant_ref.dequant(yq, fb)), torch.from_numpy(ys), padded)
+    assert torch.count_nonzero(out[2]) == 0
+    rd = gemm_ref.rdiff(out.cpu().float(), ref)
+    assert rd <= FP8_RDIFF and rd <= 2.0 ** -7, rd
+
+
+def _block_scaled_case(sizes, N, K, seed):
+    padded = [(s + 127) // 128 * 128 for s in sizes]
+    Mp, G = sum(padded), len(sizes)
+    a = to_np_f32(_randn((Mp, K), seed))
+    w = to_np_f32(_randn((G, N, K), seed + 1))
+    aq, sa = quant_ref.per_token_cast_to_fp8(a)
+    wq = np.zeros((G, N, K), np.uint8)
+    sb = np.zeros((G, (N + 127) // 128, K // 128), np.float32)
+    for g in range(G):
+        wq[g], sb[g] = quant_ref.per_block_cast_to_fp8(w[g])
+    return padded, aq, sa, wq, sb
+
+
+@pytest.mark.parametrize("sizes,N,K", [([128, 0, 100, 300], 256, 512), ([5], 200, 128), ([256, 256], 384, 1024)])
+def test_fp8_block_scaled(dev, variant, sizes, N, K):
+    """BASELINE config 5 recipe at small size: 1x128 activation scales, 128x128 weight scales, bf16 out,
+    compared with the fp32 matmul of the dequantised operands."""
+    padded, aq, sa, wq, sb = _block_scaled_case(sizes, N, K, 60)
+    Mp = sum(padded)
+    out = torch.full((Mp, N), 9.0, dtype=torch.bfloat16, device=dev)
+    ret = m_grouped_fp8_nt_contiguous((_codes_to_torch(aq, "e4m3fn").to(dev), torch.from_numpy(sa).to(dev)),
+                                      (_codes_to_torch(wq, "e4m3fn").to(dev), torch.from_numpy(sb).to(dev)),
+                                      torch.tensor(sizes, dtype=torch.int32, device=dev), out=out)
+    assert ret is out
+    ref = gemm_ref.fp8_block_scaled_reference(torch.from_numpy(quant_ref.dequant(aq)), torch.from_numpy(sa),
+                                              torch.from_numpy(quant_ref.dequant(wq)), torch.from_numpy(sb), sizes)
+    out = out.cpu().float()
+    start = 0
+    for s, p in zip(sizes, padded):
+        assert torch.equal(out[start + s:start + p], torch.full((p - s, N), 9.0))  # pad rows untouched
+        out[start + s:start + p] = 0
+        start += p
+    rd = gemm_ref.rdiff(out, ref)
+    assert rd <= FP8_RDIFF and rd <= 2.0 ** -7, rd
+
+
+def test_fp8_block_scaled_exact_with_power_of_two_scales(dev, variant):
+    """Small-integer codes and power-of-two scales: every product and partial sum is exact, so the
+    kernel must reproduce the closed form bit for bit (pins the scale indexing: a swapped or
+    transposed scale changes the answer)."""
+    g = torch.Generator().manual_seed(70)
+    sizes = [100, 128, 28]
+    padded = [128, 128, 128]
+    Mp, N, K, G = 384, 256, 384, 3
+    aq = torch.randint(-3, 4, (Mp, K), generator=g).float()
+    bq = torch.randint(-3, 4, (G, N, K), generator=g).float()
+    pw = torch.tensor([0.25, 0.5, 1.0, 2.0])
+    sa = pw[torch.randint(0, 4, (Mp, K // 128), generator=g)]
+    sb = pw[torch.randint(0, 4, (G, N // 128, K // 128), generator=g)]
+    out = m_grouped_fp8_nt_contiguous((aq.to(torch.float8_e4m3fn).to(dev), sa.to(dev)),
+                                      (bq.to(torch.float8_e4m3fn).to(dev), sb.to(dev)),
+                                      torch.tensor(sizes, dtype=torch.int32, device=dev))
+    ref = gemm_ref.fp8_block_scaled_reference(aq, sa, bq, sb, sizes)
+    assert torch.equal(ref, ref.to(torch.bfloat16).float())
+    out = out.cpu().float()
+    start = 0
+    for s, p in zip(sizes, padded):
+        assert torch.equal(out[start:start + s], ref[start:start + s])
+        start += p

@@ -1,0 +1,77 @@
+"""CPU: the product's gemm.layout helpers against the reference's known answers
+(tests/test_layout_backend.py:22-52), the plain-Python oracle, and the dtype rules."""
+import pytest
+import torch
+from hypothesis import given, settings, strategies as st
+
+from oracle import layout_ref
+from triton_grouped_gemm_amd.gemm import layout as L
+
+
+def test_round_up_to_alignment():
+    sizes = torch.tensor([0, 1, 127, 128, 129], dtype=torch.int32)
+    assert L.round_up_to_alignment(sizes, 128).tolist() == [0, 128, 128, 128, 256]
+    with pytest.raises(ValueError, match="alignment must be positive"):
+        L.round_up_to_alignment(sizes, 0)
+
+
+def test_make_group_starts_logical_and_padded():
+    sizes = torch.tensor([3, 5, 0, 7], dtype=torch.int32)
+    assert L.make_group_starts(sizes, padded=False, block_m=4).tolist() == [0, 3, 8, 8]
+    assert L.make_group_starts(sizes, padded=True, block_m=4).tolist() == [0, 4, 12, 12]
+
+
+def test_make_grouped_layout_summary_and_dtypes():
+    lay = L.make_grouped_layout([3, 5, 0, 7], block_m=4)
+    assert lay.sizes.tolist() == [3, 5, 0, 7]
+    assert lay.padded_sizes.tolist() == [4, 8, 0, 8]
+    assert lay.starts.tolist() == [0, 4, 12, 12]
+    assert int(lay.total_m.item()) == 15 and int(lay.total_padded_m.item()) == 20
+    # cumsum of int32 is int64 in torch; the reference's starts therefore are int64
+    assert lay.sizes.dtype == torch.int32 and lay.padded_sizes.dtype == torch.int32
+    assert lay.starts.dtype == torch.int64 and lay.total_m.dtype == torch.int64
+    assert L.make_group_starts([1, 2]).dtype == torch.int64
+
+
+def test_deep_gemm_layouts():
+    assert L.make_deep_gemm_grouped_layout([3, 5], block_m=4).tolist() == [0, 0, 0, -1, 1, 1, 1, 1, 1, -1, -1, -1]
+    assert L.make_deep_gemm_psum_layout([3, 5], block_m=4).tolist() == [3, 9]
+    assert L.make_deep_gemm_grouped_layout([3, 5], block_m=4).dtype == torch.int32
+    assert L.make_deep_gemm_psum_layout([3, 5], block_m=4).dtype == torch.int32
+    assert L.make_deep_gemm_grouped_layout([0, 0]).numel() == 0
+
+
+def test_validate_total_m_and_size_checks():
+    L.validate_total_m([2, 3, 4], 9)
+    with pytest.raises(ValueError, match=r"sum\(size_per_group\)"):
+        L.validate_total_m([2, 3, 4], 10)
+    with pytest.raises(ValueError, match="1D"):
+        L.as_group_sizes(torch.zeros(2, 2, dtype=torch.int32))
+    with pytest.raises(ValueError, match="at least one group"):
+        L.as_group_sizes([])
+    with pytest.raises(ValueError, match="negative"):
+        L.as_group_sizes([1, -1])
+    assert L.as_group_sizes(torch.tensor([1, 2], dtype=torch.int64)).dtype == torch.int32
+
+
+@settings(max_examples=60, deadline=None)
+@given(st.lists(st.integers(0, 700), min_size=1, max_size=40), st.sampled_from([1, 4, 64, 128]))
+def test_layout_matches_plain_python_oracle(sizes, block_m):
+    assert L.make_group_starts(sizes, padded=False, block_m=block_m).tolist() == layout_ref.group_starts(sizes, False, block_m)
+    assert L.make_group_starts(sizes, padded=True, block_m=block_m).tolist() == layout_ref.group_starts(sizes, True, block_m)
+    ref = layout_ref.grouped_layout(sizes, block_m)
+    lay = L.make_grouped_layout(sizes, block_m)
+    assert lay.starts.tolist() == ref["starts"] and lay.padded_sizes.tolist() == ref["padded_sizes"]
+    assert L.make_deep_gemm_grouped_layout(sizes, block_m=block_m).tolist() == layout_ref.deep_gemm_grouped_layout(sizes, block_m)
+    assert L.make_deep_gemm_psum_layout(sizes, block_m=block_m).tolist() == layout_ref.deep_gemm_psum_layout(sizes, block_m)
+
+
+def test_metadata_builder_matches_oracle():
+    from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm import _build_m_grouped_metadata
+    sizes = [3, 0, 130, 128, 1, 257]
+    ps, pe, gs, ge, idx, mpad = _build_m_grouped_metadata(torch.tensor(sizes, dtype=torch.int32))
+    rps, rpe, rgs, rge, ridx, rmpad = layout_ref.m_grouped_metadata(sizes)
+    assert ps.tolist() == rps and pe.tolist() == rpe and gs.tolist() == rgs and ge.tolist() == rge
+    assert idx[: len(ridx)].tolist() == ridx and int(mpad) == rmpad
+    assert idx.numel() == sum(sizes) // 128 + len(sizes) and idx.dtype == torch.int32
+    assert ps.dtype == torch.int32 and gs.dtype == torch.int64

@@ -1,0 +1,208 @@
+"""CPU: pin the oracle (tests' checker) against the reference's known answers, library
+routines and brute force, so that a wrong index / sign / dropped term in it fails here."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8_soft, gemm_ref, layout_ref, quant_ref
+
+
+# ---- layout: the reference's own known answers (tests/test_layout_backend.py:23-52) ----
+def test_layout_known_answers():
+    assert layout_ref.round_up([0, 1, 127, 128, 129], 128) == [0, 128, 128, 128, 256]
+    assert layout_ref.group_starts([3, 5, 0, 7], padded=False, block_m=4) == [0, 3, 8, 8]
+    assert layout_ref.group_starts([3, 5, 0, 7], padded=True, block_m=4) == [0, 4, 12, 12]
+    lay = layout_ref.grouped_layout([3, 5, 0, 7], block_m=4)
+    assert lay["sizes"] == [3, 5, 0, 7] and lay["padded_sizes"] == [4, 8, 0, 8]
+    assert lay["starts"] == [0, 4, 12, 12] and lay["total_m"] == 15 and lay["total_padded_m"] == 20
+    assert layout_ref.deep_gemm_grouped_layout([3, 5], 4) == [0, 0, 0, -1, 1, 1, 1, 1, 1, -1, -1, -1]
+    assert layout_ref.deep_gemm_psum_layout([3, 5], 4) == [3, 9]
+    layout_ref.validate_total_m([2, 3, 4], 9)
+    with pytest.raises(ValueError, match=r"sum\(size_per_group\)"):
+        layout_ref.validate_total_m([2, 3, 4], 10)
+
+
+def test_tile_rows_cover_every_row_once():
+    sizes = [3, 0, 130, 128, 1, 257]
+    seen = []
+    for g, row0, rows in layout_ref.tile_rows(sizes, 128):
+        assert 0 < rows <= 128
+        seen += [(g, r) for r in range(row0, row0 + rows)]
+    want, start = [], 0
+    for g, s in enumerate(sizes):
+        want += [(g, r) for r in range(start, start + s)]
+        start += s
+    assert seen == want
+
+
+# ---- fp8 encoders: exhaustive against torch's CPU cast, and closed-form round trips ----
+def _all_bf16_as_f32():
+    return fp8_soft.bf16_bits_to_f32(np.arange(65536, dtype=np.uint16))
+
+
+@pytest.mark.parametrize("fmt,tdt,enc", [("e4m3fn", torch.float8_e4m3fn, fp8_soft.encode_e4m3fn),
+                                         ("e5m2", torch.float8_e5m2, fp8_soft.encode_e5m2)])
+def test_fp8_encode_matches_torch_cast(fmt, tdt, enc):
+    rng = np.random.default_rng(0)
+    x = np.concatenate([_all_bf16_as_f32(),
+                        (rng.standard_normal(200000) * np.exp(rng.uniform(-25, 12, 200000))).astype(np.float32),
+                        np.array([448.0, 464.0, 463.99, 465.0, 57344.0, 61440.0, 61439.0, 2.0 ** -9, 2.0 ** -10,
+                                  1.5 * 2.0 ** -10, 2.0 ** -16, 2.0 ** -17, 0.0, -0.0], dtype=np.float32)])
+    with np.errstate(all="ignore"):
+        mine = enc(x)
+    ref = torch.from_numpy(x).to(tdt).view(torch.uint8).numpy()
+    nan_mine = np.isnan(quant_ref.dequant(mine, fmt))
+    nan_ref = np.isnan(quant_ref.dequant(ref, fmt))
+    assert np.array_equal(nan_mine, nan_ref)
+    assert np.array_equal(mine[~nan_ref], ref[~nan_ref])
+
+
+def test_fp8_decode_encode_roundtrip_and_spacing():
+    codes = np.arange(256, dtype=np.uint8)
+    v = fp8_soft.decode_e4m3fn(codes)
+    ok = ~np.isnan(v)
+    assert np.array_equal(fp8_soft.encode_e4m3fn(v[ok]), codes[ok])
+    assert v[0x7E] == 448.0 and v[0x01] == 2.0 ** -9 and v[0x08] == 2.0 ** -6 and np.isnan(v[0x7F])
+    v5 = fp8_soft.decode_e5m2(codes)
+    ok5 = np.isfinite(v5)
+    assert np.array_equal(fp8_soft.encode_e5m2(v5[ok5]), codes[ok5])
+    assert v5[0x7B] == 57344.0 and v5[0x01] == 2.0 ** -16 and np.isinf(v5[0x7C])
+    # ties go to even: halfway between codes 0x40 (2.0) and 0x41 (2.25) -> 0x40; next tie -> 0x42
+    assert fp8_soft.encode_e4m3fn(np.array([2.125, 2.375], np.float32)).tolist() == [0x40, 0x42]
+
+
+def test_bf16_rounding_matches_torch():
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal(100000) * np.exp(rng.uniform(-30, 30, 100000))).astype(np.float32)
+    ref = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(fp8_soft.f32_to_bf16_bits(x), ref)
+
+
+# ---- quantizers: brute force per element on tiny inputs + invariants ----
+def _bf16_randn(shape, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(torch.bfloat16).float().numpy()
+
+
+def test_trans_quant_bruteforce_and_invariants():
+    sizes = [5, 0, 130, 128]
+    M, N = sum(sizes), 256
+    x = _bf16_randn((M, N), 3)
+    codes, scales, padded = quant_ref.trans_per_block_quant_expand_128x(x, sizes)
+    ME = M + 128 * len(sizes) - M % 128
+    assert codes.shape == (N, ME) and scales.shape == (N // 128, ME // 128)
+    assert padded.tolist() == [128, 0, 256, 128]
+    # brute force: element by element with Python scalars
+    src, dst = 0, 0
+    for s, p in zip(sizes, padded.tolist()):
+        for r in range(p):
+            for n in range(0, N, 37):
+                blk_r0 = src + (r // 128) * 128
+                blk = x[blk_r0:min(blk_r0 + 128, src + s), (n // 128) * 128:(n // 128 + 1) * 128]
+                amax = np.float32(np.abs(blk).max()) if blk.size else np.float32(0)
+                sc = np.float32(max(np.float32(amax / np.float32(448.0)), np.float32(1e-12)))
+                assert scales[n // 128, (dst + r) // 128] == sc
+                val = x[src + r, n] if r < s else np.float32(0)
+                q = np.float32(min(max(np.float32(val / sc), -448.0), 448.0))
+                want = torch.tensor([q]).to(torch.float8_e4m3fn).view(torch.uint8).item()
+                assert codes[n, dst + r] == want
+        src += s
+        dst += p
+    # tail beyond the padded groups is zero
+    assert not codes[:, dst:].any() and not scales[:, dst // 128:].any()
+    # dequantised codes sit within half an e4m3 ulp (2^-4 relative of the block max) of x
+    deq = quant_ref.dequant(codes[:, :128], "e4m3fn") * scales[:, 0:1].repeat(128, axis=0)
+    err = np.abs(deq[:, :5].T - x[:5])
+    assert err.max() <= np.abs(x[:5]).max() * 2.0 ** -4
+
+
+def test_trans_quant_matches_reference_torch_oracle_on_full_blocks():
+    """The reference's own torch oracle (quant/...:222-273) restated inline with torch ops."""
+    sizes = [128, 256]
+    M, N = 384, 128
+    x = _bf16_randn((M, N), 4)
+    codes, scales, _ = quant_ref.trans_per_block_quant_expand_128x(x, sizes)
+    xt = torch.from_numpy(x).to(torch.bfloat16)
+    outs, scs = [], []
+    for part in torch.split(xt, sizes, dim=0):
+        t = part.T
+        d, s = t.shape
+        blocks = t.reshape(d // 128, 128, s // 128, 128).transpose(1, 2).reshape(-1, 128 * 128)
+        sc = blocks.abs().amax(-1, True).float() / 448.0
+        q = (blocks / sc).clamp(-448, 448).to(torch.float8_e4m3fn)
+        outs.append(q.reshape(d // 128, s // 128, 128, 128).transpose(1, 2).reshape(d, s))
+        scs.append(sc.reshape(d // 128, s // 128))
+    ref_codes = torch.cat(outs, -1).view(torch.uint8).numpy()
+    ref_scales = torch.cat(scs, -1).numpy()
+    assert np.array_equal(codes[:, :M], ref_codes)
+    assert np.array_equal(scales[:, :M // 128], ref_scales)
+
+
+def test_cast_recipes_match_torch_expressions():
+    x = _bf16_randn((16, 256), 5, scale=3.0)
+    xt = torch.from_numpy(x).to(torch.bfloat16)
+    codes, scales = quant_ref.per_token_cast_to_fp8(x)
+    v = xt.view(16, -1, 128)
+    amax = v.abs().float().amax(dim=2).view(16, -1).clamp(1e-4)
+    ref = (v * (448.0 / amax.unsqueeze(2))).to(torch.float8_e4m3fn).view(16, 256).view(torch.uint8).numpy()
+    assert np.array_equal(codes, ref) and np.array_equal(scales, (amax / 448.0).numpy())
+    xb = _bf16_randn((130, 200), 6)
+    cb, sb = quant_ref.per_block_cast_to_fp8(xb)
+    assert cb.shape == (130, 200) and sb.shape == (2, 2)
+    blk = xb[128:, 128:]
+    assert sb[1, 1] == np.float32(np.float32(np.abs(blk).max()) / np.float32(448.0))
+    # a block of zeros hits the 1e-4 clamp
+    cz, sz = quant_ref.per_block_cast_to_fp8(np.zeros((128, 128), np.float32))
+    assert sz[0, 0] == np.float32(np.float32(1e-4) / np.float32(448.0)) and not cz.any()
+
+
+# ---- GEMM references: reduce to library routines ----
+def test_gmm_reduces_to_matmul_and_bmm():
+    g = torch.Generator().manual_seed(7)
+    a = torch.randn(96, 32, generator=g)
+    b = torch.randn(3, 48, 32, generator=g)
+    assert torch.equal(gemm_ref.gmm(a, b[:1], [96], trans_b=True), a @ b[0].t())
+    out = gemm_ref.gmm(a, b, [32, 32, 32], trans_b=True)
+    assert torch.allclose(out.view(3, 32, 48), torch.bmm(a.view(3, 32, 32), b.transpose(1, 2)), atol=1e-5)
+    bn = b.transpose(1, 2).contiguous()
+    assert torch.allclose(gemm_ref.gmm(a, bn, [10, 0, 86], trans_b=False), gemm_ref.gmm(a, b, [10, 0, 86], trans_b=True), atol=1e-5)
+    # permuting experts permutes output blocks
+    perm = gemm_ref.gmm(torch.cat([a[64:], a[:64]]), b[[2, 0, 1]], [32, 32, 32], trans_b=True)
+    assert torch.allclose(perm[:32], out[64:], atol=1e-6)
+
+
+def test_gmm_dw_and_masked_special_cases():
+    g = torch.Generator().manual_seed(8)
+    a = torch.randn(40, 16, generator=g)
+    b = torch.randn(40, 24, generator=g)
+    assert torch.allclose(gemm_ref.gmm_dw(a, b, [40])[0], a.t() @ b, atol=1e-5)
+    out = gemm_ref.gmm_dw(a, b, [10, 0, 30])
+    assert torch.count_nonzero(out[1]) == 0
+    assert torch.allclose(out[0] + out[2], a.t() @ b, atol=1e-4)
+    lhs = torch.randn(4 * 8, 16, generator=g)
+    rhs = torch.randn(4, 12, 16, generator=g)
+    outs = gemm_ref.masked_gmm(lhs, rhs, [8, 8, 8, 8], 8)
+    assert torch.allclose(torch.stack(outs), torch.bmm(lhs.view(4, 8, 16), rhs.transpose(1, 2)), atol=1e-5)
+    assert gemm_ref.masked_gmm(lhs, rhs, [0, 3, 8, 1], 8)[1].shape == (3, 12)
+
+
+def test_block_scaled_reference_exact_on_power_of_two_scales():
+    g = torch.Generator().manual_seed(9)
+    sizes = [100, 128]
+    Mp, K, N = 256, 256, 128
+    aq = torch.randint(-4, 5, (Mp, K), generator=g).float()
+    bq = torch.randint(-4, 5, (2, N, K), generator=g).float()
+    sa = torch.tensor([0.5, 2.0]).repeat(Mp, 1)
+    sb = torch.tensor([4.0, 0.25]).view(1, 1, 2).repeat(2, 1, 1)
+    out = gemm_ref.fp8_block_scaled_reference(aq, sa, bq, sb, sizes)
+    want0 = 2.0 * (aq[:100, :128] @ bq[0][:, :128].t()) + 0.5 * (aq[:100, 128:] @ bq[0][:, 128:].t())
+    assert torch.equal(out[:100], want0)
+    assert torch.count_nonzero(out[100:128]) == 0
+    assert torch.equal(out[128:], 2.0 * (aq[128:, :128] @ bq[1][:, :128].t()) + 0.5 * (aq[128:, 128:] @ bq[1][:, 128:].t()))
+
+
+def test_metrics():
+    x = torch.tensor([1.0, -2.0, 4.0])
+    assert gemm_ref.rdiff(x, x) == 0.0 and gemm_ref.cos_diff(x, x) == pytest.approx(0.0, abs=1e-15)
+    assert gemm_ref.rdiff(x, x + torch.tensor([0.0, 0.0, 0.4])) == pytest.approx(0.4 / 4.4)
+    assert torch.allclose(gemm_ref.row_max_normalization(torch.tensor([[1.0, -4.0]])), torch.tensor([[0.25, -1.0]]))

@@ -1,0 +1,88 @@
+"""ctypes binding of libtgg_amd.so (the C ABI declared in include/tgg_amd.h).
+
+There is no fallback: if the shared library is missing or a call fails, the
+caller gets an exception.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_int, c_int64, c_void_p
+from pathlib import Path
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "libtgg_amd.so"
+
+BF16, F16, E4M3, E5M2 = 0, 1, 2, 3
+MAX_GROUPS = 1024
+
+_P, _I, _L = c_void_p, c_int, c_int64
+
+# name -> argument types; every function returns int unless noted
+SIGNATURES = {
+    "tgg_m_grouped_gemm": [_P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _I, _P],
+    "tgg_m_grouped_gemm_padded": [_P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _I, _P],
+    "tgg_m_grouped_gemm_masked": [_P, _P, _P, _P, _I, _I, _L, _L, _I, _I, _I, _I, _I, _P],
+    "tgg_k_grouped_gemm": [_P, _P, _P, _P, _P, _I, _I, _I, _L, _I, _I, _P],
+    "tgg_m_grouped_gemm_fp8_channel": [_P, _P, _P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _I, _I, _P],
+    "tgg_k_grouped_gemm_fp8_channel": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _L, _I, _I, _I, _P],
+    "tgg_m_grouped_gemm_fp8_block": [_P, _P, _P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _P],
+    "tgg_trans_per_block_quant_expand_128x": [_P, _P, _P, _P, _I, _I, _L, _I, _L, _I, _P],
+    "tgg_per_token_cast_to_fp8": [_P, _P, _P, _L, _I, _I, _P],
+    "tgg_per_block_cast_to_fp8": [_P, _P, _P, _I, _I, _I, _I, _P],
+    "tgg_cvt_f32_to_fp8": [_P, _P, _L, _I, _P],
+    "tgg_set_option": [c_char_p, _I],
+    "tgg_version": [],
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m triton_grouped_gemm_amd.build` "
+                "(there is no non-HIP fallback)")
+        lib = ctypes.CDLL(str(LIB_PATH))
+        for name, args in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = args
+            fn.restype = c_int
+        lib.tgg_last_error.argtypes = []
+        lib.tgg_last_error.restype = c_char_p
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    return load().tgg_last_error().decode()
+
+
+def call(name: str, *args) -> None:
+    rc = getattr(load(), name)(*args)
+    if rc != 0:
+        raise RuntimeError(f"{name} failed (code {rc}): {last_error()}")
+
+
+def set_option(key: str, value: int) -> None:
+    call("tgg_set_option", key.encode(), int(value))
+
+
+def stream_of(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def ptr(t) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def require_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise AssertionError("all tensors must live on the GPU (HIP device); this library has no CPU path")
+
+
+DTYPE_CODE = {torch.bfloat16: BF16, torch.float16: F16}
+FP8_CODE = {torch.float8_e4m3fn: E4M3, torch.float8_e5m2: E5M2}

@@ -1,0 +1,240 @@
+// extern "C" surface of libtgg_amd.so: argument validation, GemmParams assembly, dispatch.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/tgg_amd.h"
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace tgg {
+
+static thread_local char g_err[512] = "";
+static int g_force_generic = 0;
+
+int set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return 1;
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return 0;
+  snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(e));
+  return 2;
+}
+
+int num_cus() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+int launch_trans_quant128(const void*, void*, float*, const GemmParams&, int64_t, int, hipStream_t);
+int launch_token_cast128(const void*, void*, float*, int64_t, int, hipStream_t);
+int launch_block_cast128(const void*, void*, float*, int, int, int, int, hipStream_t);
+int launch_cvt_fp8(const float*, void*, int64_t, int, hipStream_t);
+bool fast_supported(const GemmParams& p, int dt, int layout);
+int launch_fast_16bit(const GemmParams& p, int dt, int layout, hipStream_t s);
+
+static bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
+
+static int check_common(const void* A, const void* B, const void* C, const void* sizes, int G, int N) {
+  if (!A || !B || !C) return set_error("null operand pointer");
+  if (!sizes) return set_error("null group-size pointer");
+  if (G < 1 || G > TGG_MAX_GROUPS) return set_error("G=%d outside [1, %d]", G, TGG_MAX_GROUPS);
+  if (N < 1) return set_error("N=%d must be positive", N);
+  if (!aligned16(A) || !aligned16(B) || !aligned16(C)) return set_error("operand pointers must be 16-byte aligned");
+  return 0;
+}
+
+static GemmParams zero_params() {
+  GemmParams p;
+  memset(&p, 0, sizeof(p));
+  return p;
+}
+
+static int dispatch_16bit(const GemmParams& p, int dt, int layout, hipStream_t s) {
+  if (!g_force_generic && fast_supported(p, dt, layout)) return launch_fast_16bit(p, dt, layout, s);
+  return launch_generic_16bit(p, dt, layout, s);
+}
+
+}  // namespace tgg
+
+using namespace tgg;
+
+extern "C" {
+
+int tgg_m_grouped_gemm(const void* A, const void* B, void* C, const void* sizes, int sizes_i64, int G, int64_t M,
+                       int N, int K, int trans_b, int dtype, int num_cu, void* stream) {
+  if (int e = check_common(A, B, C, sizes, G, N)) return e;
+  if (M < 0 || K < 0) return set_error("negative M or K");
+  if (dtype != TGG_BF16 && dtype != TGG_F16) return set_error("data type code %d not supported", dtype);
+  if ((K & 7) || (N & 7)) return set_error("N and K must be multiples of 8 (16-byte rows), got N=%d K=%d", N, K);
+  if (M == 0) return 0;
+  GemmParams p = zero_params();
+  p.A = A; p.B = B; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
+  p.mode = MODE_MG; p.m_total = M; p.N = N; p.K = K;
+  p.a_sm = K; p.a_sk = 1;
+  p.b_sg = (int64_t)N * K;
+  if (trans_b) { p.b_sn = K; p.b_sk = 1; } else { p.b_sn = 1; p.b_sk = N; }
+  p.grid_limit = num_cu;
+  return dispatch_16bit(p, dtype, trans_b ? 0 : 1, (hipStream_t)stream);
+}
+
+int tgg_m_grouped_gemm_padded(const void* A, const void* B, void* C, const void* sizes, int sizes_i64, int G,
+                              int64_t M, int N, int K, int align, int dtype, int num_cu, void* stream) {
+  if (int e = check_common(A, B, C, sizes, G, N)) return e;
+  if (M < 0 || K < 0) return set_error("negative M or K");
+  if (align < 1) return set_error("alignment must be positive, got %d", align);
+  if (dtype != TGG_BF16 && dtype != TGG_F16) return set_error("data type code %d not supported", dtype);
+  if ((K & 7) || (N & 7)) return set_error("N and K must be multiples of 8 (16-byte rows), got N=%d K=%d", N, K);
+  if (M == 0) return 0;
+  GemmParams p = zero_params();
+  p.A = A; p.B = B; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
+  p.mode = MODE_MG_PAD; p.align = align; p.m_total = M; p.N = N; p.K = K;
+  p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K; p.b_sn = K; p.b_sk = 1;
+  p.grid_limit = num_cu;
+  return dispatch_16bit(p, dtype, 0, (hipStream_t)stream);
+}
+
+int tgg_m_grouped_gemm_masked(const void* A, const void* B, void* C, const void* masked_m, int masked_i64, int G,
+                              int64_t m_stride, int64_t M, int N, int K, int trans_b, int dtype, int num_cu,
+                              void* stream) {
+  if (int e = check_common(A, B, C, masked_m, G, N)) return e;
+  if (M < 0 || K < 0 || m_stride < 0) return set_error("negative M, K or m_stride");
+  if (dtype != TGG_BF16 && dtype != TGG_F16) return set_error("data type code %d not supported", dtype);
+  if ((K & 7) || (N & 7)) return set_error("N and K must be multiples of 8 (16-byte rows), got N=%d K=%d", N, K);
+  if (M == 0 || m_stride == 0) return 0;
+  GemmParams p = zero_params();
+  p.A = A; p.B = B; p.C = C; p.sizes = masked_m; p.sizes_i64 = masked_i64; p.G = G;
+  p.mode = MODE_MASKED; p.m_stride = m_stride; p.m_total = M; p.N = N; p.K = K;
+  p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K;
+  if (trans_b) { p.b_sn = K; p.b_sk = 1; } else { p.b_sn = 1; p.b_sk = N; }
+  p.grid_limit = num_cu;
+  return dispatch_16bit(p, dtype, trans_b ? 0 : 1, (hipStream_t)stream);
+}
+
+int tgg_k_grouped_gemm(const void* A, const void* B, void* C, const int32_t* start, const int32_t* end, int G,
+                       int Mdim, int N, int64_t Ktot, int dtype, int num_cu, void* stream) {
+  if (int e = check_common(A, B, C, start, G, N)) return e;
+  if (!end) return set_error("null group_end pointer");
+  if (Mdim < 1 || Ktot < 0) return set_error("bad Mdim=%d or Ktot=%lld", Mdim, (long long)Ktot);
+  if (dtype != TGG_BF16 && dtype != TGG_F16) return set_error("data type code %d not supported", dtype);
+  if ((Mdim & 7) || (N & 7)) return set_error("Mdim and N must be multiples of 8 (16-byte rows), got %d, %d", Mdim, N);
+  GemmParams p = zero_params();
+  p.A = A; p.B = B; p.C = C; p.k_start = start; p.k_end = end; p.G = G;
+  p.mode = MODE_KG; p.m_total = Mdim; p.N = N; p.K = 0;
+  p.a_sm = 1; p.a_sk = Mdim; p.b_sg = 0; p.b_sn = 1; p.b_sk = N; p.c_sg = (int64_t)Mdim * N;
+  p.grid_limit = num_cu;
+  return dispatch_16bit(p, dtype, 2, (hipStream_t)stream);
+}
+
+static bool is_fp8(int f) { return f == TGG_E4M3 || f == TGG_E5M2; }
+
+int tgg_m_grouped_gemm_fp8_channel(const void* Aq, const float* a_scale, const void* Bq, const float* b_scale,
+                                   void* C, const void* sizes, int sizes_i64, int G, int64_t M, int N, int K,
+                                   int fmt_a, int fmt_b, int out_dtype, int num_cu, void* stream) {
+  if (int e = check_common(Aq, Bq, C, sizes, G, N)) return e;
+  if (!a_scale || !b_scale) return set_error("null scale pointer");
+  if (M < 0 || K < 0) return set_error("negative M or K");
+  if (!is_fp8(fmt_a) || !is_fp8(fmt_b)) return set_error("fp8 format codes must be E4M3 or E5M2");
+  if (K & 15) return set_error("K must be a multiple of 16 for fp8 operands, got %d", K);
+  if (M == 0) return 0;
+  GemmParams p = zero_params();
+  p.A = Aq; p.B = Bq; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
+  p.scale_m = a_scale; p.scale_n = b_scale;
+  p.mode = MODE_MG; p.m_total = M; p.N = N; p.K = K;
+  p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K; p.b_sn = K; p.b_sk = 1;
+  p.grid_limit = num_cu;
+  return launch_generic_fp8_channel(p, fmt_a, fmt_b, out_dtype, (hipStream_t)stream);
+}
+
+int tgg_k_grouped_gemm_fp8_channel(const void* x, const float* xs, const void* y, const float* ys, void* out,
+                                   const int32_t* tokens, int G, int M, int N, int64_t Ktot, int fmt_a, int fmt_b,
+                                   int num_cu, void* stream) {
+  if (int e = check_common(x, y, out, tokens, G, N)) return e;
+  if (!xs || !ys) return set_error("null scale pointer");
+  if (M < 1 || Ktot < 0) return set_error("bad M=%d or Ktot=%lld", M, (long long)Ktot);
+  if (!is_fp8(fmt_a) || !is_fp8(fmt_b)) return set_error("fp8 format codes must be E4M3 or E5M2");
+  if (Ktot & 15) return set_error("Ktot must be a multiple of 16 for fp8 operands, got %lld", (long long)Ktot);
+  GemmParams p = zero_params();
+  p.A = x; p.B = y; p.C = out; p.sizes = tokens; p.sizes_i64 = 0; p.G = G;
+  p.scale_m = xs; p.scale_n = ys; p.scale_m_sg = M;
+  p.mode = MODE_KG_COUNT; p.m_total = M; p.N = N; p.K = 0;
+  p.a_sm = Ktot; p.a_sk = 1; p.b_sg = 0; p.b_sn = Ktot; p.b_sk = 1; p.c_sg = (int64_t)M * N;
+  p.grid_limit = num_cu;
+  return launch_generic_fp8_channel(p, fmt_a, fmt_b, TGG_BF16, (hipStream_t)stream);
+}
+
+int tgg_m_grouped_gemm_fp8_block(const void* Aq, const float* sa, const void* Bq, const float* sb, void* C,
+                                 const void* sizes, int sizes_i64, int G, int64_t M, int N, int K, int align,
+                                 int num_cu, void* stream) {
+  if (int e = check_common(Aq, Bq, C, sizes, G, N)) return e;
+  if (!sa || !sb) return set_error("null scale pointer");
+  if (M < 0 || K < 0) return set_error("negative M or K");
+  if (align < 1 || (align & 127)) return set_error("alignment must be a positive multiple of 128, got %d", align);
+  if (K & 15) return set_error("K must be a multiple of 16 for fp8 operands, got %d", K);
+  if (M == 0) return 0;
+  GemmParams p = zero_params();
+  p.A = Aq; p.B = Bq; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
+  p.sa = sa; p.sb = sb;
+  p.mode = MODE_MG_PAD; p.align = align; p.m_total = M; p.N = N; p.K = K;
+  p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K; p.b_sn = K; p.b_sk = 1;
+  p.grid_limit = num_cu;
+  return launch_generic_fp8_block(p, (hipStream_t)stream);
+}
+
+int tgg_trans_per_block_quant_expand_128x(const void* x, void* codes, float* scales, const void* sizes,
+                                          int sizes_i64, int G, int64_t M, int N, int64_t M_expand, int fmt,
+                                          void* stream) {
+  if (!x || !codes || !scales || !sizes) return set_error("null pointer");
+  if (G < 1 || G > TGG_MAX_GROUPS) return set_error("G=%d outside [1, %d]", G, TGG_MAX_GROUPS);
+  if (N < 128 || (N & 127)) return set_error("N must be a positive multiple of 128, got %d", N);
+  if (M < 0 || M_expand < 0 || (M_expand & 127)) return set_error("M_expand must be a multiple of 128");
+  if (M_expand < ((M + 127) / 128) * 128) return set_error("M_expand=%lld too small for M=%lld", (long long)M_expand, (long long)M);
+  if (!aligned16(x) || !aligned16(codes)) return set_error("operand pointers must be 16-byte aligned");
+  if (M_expand == 0) return 0;
+  GemmParams p = zero_params();
+  p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G; p.mode = MODE_MG; p.m_total = M; p.N = N;
+  return launch_trans_quant128(x, codes, scales, p, M_expand, fmt, (hipStream_t)stream);
+}
+
+int tgg_per_token_cast_to_fp8(const void* x, void* codes, float* scales, int64_t M, int K, int fmt, void* stream) {
+  if (!x || !codes || !scales) return set_error("null pointer");
+  if (M < 0 || K < 0 || (K & 127)) return set_error("K must be a multiple of 128, got %d", K);
+  if (!aligned16(x) || !aligned16(codes)) return set_error("operand pointers must be 16-byte aligned");
+  return launch_token_cast128(x, codes, scales, M * (K / 128), fmt, (hipStream_t)stream);
+}
+
+int tgg_per_block_cast_to_fp8(const void* x, void* codes, float* scales, int batch, int R, int C, int fmt,
+                              void* stream) {
+  if (!x || !codes || !scales) return set_error("null pointer");
+  if (batch < 0 || R < 0 || C < 0) return set_error("negative shape");
+  if (!aligned16(x) || !aligned16(codes)) return set_error("operand pointers must be 16-byte aligned");
+  return launch_block_cast128(x, codes, scales, batch, R, C, fmt, (hipStream_t)stream);
+}
+
+int tgg_cvt_f32_to_fp8(const float* in, void* out, int64_t n, int fmt, void* stream) {
+  if (!in || !out || n < 0) return set_error("bad arguments");
+  return launch_cvt_fp8(in, out, n, fmt, (hipStream_t)stream);
+}
+
+int tgg_set_option(const char* key, int value) {
+  if (key && strcmp(key, "force_generic") == 0) { g_force_generic = value != 0; return 0; }
+  return set_error("unknown option '%s'", key ? key : "(null)");
+}
+
+const char* tgg_last_error(void) { return g_err; }
+int tgg_version(void) { return 100; }
+
+}  // extern "C"

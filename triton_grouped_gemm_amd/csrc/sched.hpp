@@ -1,0 +1,131 @@
+// Per-workgroup tile scheduler for grouped GEMMs.
+//
+// Every workgroup rebuilds the same small table in LDS from the per-group sizes
+// (an exclusive prefix sum of rows and of M-tiles) and then walks the tile space
+// with a persistent, XCD-aware stride.  No host-side metadata, no workspace, no
+// host/device synchronisation.
+#pragma once
+#include "common.hpp"
+
+namespace tgg {
+
+constexpr int kMaxGroups = 1024;
+
+struct SchedTable {
+  int64_t row0[kMaxGroups];     // first row of the group in A/C (M modes) or first k (K modes)
+  int32_t rows[kMaxGroups];     // valid rows (M modes) or k extent (K modes)
+  int32_t tile0[kMaxGroups + 1];// exclusive prefix of ceil(rows / BM) (M modes only)
+};
+
+struct Tile {
+  int g;
+  int64_t row0;   // first row of this tile in A and C (M modes); first m within the group (K modes)
+  int rows;       // valid rows in this tile (<= BM)
+  int n0;
+  int64_t k0;     // reduction range [k0, k1)
+  int64_t k1;
+};
+
+TGG_DEV int64_t load_size(const void* p, int is64, int i) {
+  int64_t v = is64 ? ((const int64_t*)p)[i] : (int64_t)((const int32_t*)p)[i];
+  return v < 0 ? 0 : v;
+}
+
+// All threads of the workgroup must call this; ends with a barrier.
+template <int BM>
+TGG_DEV void sched_init(const GemmParams& p, SchedTable& t) {
+  const int G = p.G;
+  if (p.mode == MODE_KG) {
+    for (int g = threadIdx.x; g < G; g += blockDim.x) {
+      int64_t s = p.k_start[g], e = p.k_end[g];
+      t.row0[g] = s;
+      t.rows[g] = e > s ? (int32_t)(e - s) : 0;
+    }
+    __syncthreads();
+    return;
+  }
+  for (int g = threadIdx.x; g < G; g += blockDim.x) t.rows[g] = (int32_t)load_size(p.sizes, p.sizes_i64, g);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int64_t row = 0;
+    int32_t tile = 0;
+    for (int g = 0; g < G; ++g) {
+      int64_t sz = t.rows[g];
+      int64_t start;
+      if (p.mode == MODE_MASKED) {
+        start = (int64_t)g * p.m_stride;
+        if (sz > p.m_stride) sz = p.m_stride;
+      } else {
+        start = row;
+        row += (p.mode == MODE_MG_PAD) ? ((sz + p.align - 1) / p.align) * p.align : sz;
+      }
+      if (p.mode != MODE_KG_COUNT) {  // never touch rows past the end of A / C
+        if (start >= p.m_total) sz = 0;
+        else if (start + sz > p.m_total) sz = p.m_total - start;
+      }
+      t.row0[g] = start;
+      t.rows[g] = (int32_t)sz;
+      t.tile0[g] = tile;
+      tile += (int32_t)((sz + BM - 1) / BM);
+    }
+    t.tile0[G] = tile;
+  }
+  __syncthreads();
+}
+
+template <int BM, int BN>
+TGG_DEV int64_t sched_num_tiles(const GemmParams& p, const SchedTable& t) {
+  const int tiles_n = (p.N + BN - 1) / BN;
+  if (p.mode == MODE_KG || p.mode == MODE_KG_COUNT) {
+    const int tiles_m = (int)((p.m_total + BM - 1) / BM);
+    return (int64_t)p.G * tiles_m * tiles_n;
+  }
+  return (int64_t)t.tile0[p.G] * tiles_n;
+}
+
+template <int BM, int BN>
+TGG_DEV Tile sched_tile(const GemmParams& p, const SchedTable& t, int64_t tile_id) {
+  Tile r;
+  const int tiles_n = (p.N + BN - 1) / BN;
+  if (p.mode == MODE_KG || p.mode == MODE_KG_COUNT) {
+    const int tiles_m = (int)((p.m_total + BM - 1) / BM);
+    const int per_group = tiles_m * tiles_n;
+    r.g = (int)(tile_id / per_group);
+    const int rem = (int)(tile_id % per_group);
+    const int mt = rem / tiles_n;
+    r.n0 = (rem % tiles_n) * BN;
+    r.row0 = (int64_t)mt * BM;
+    const int64_t left = p.m_total - r.row0;
+    r.rows = left < BM ? (int)left : BM;
+    r.k0 = t.row0[r.g];
+    r.k1 = r.k0 + t.rows[r.g];
+    return r;
+  }
+  const int mt_glob = (int)(tile_id / tiles_n);
+  r.n0 = (int)(tile_id % tiles_n) * BN;
+  int lo = 0, hi = p.G;  // last g with tile0[g] <= mt_glob
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (t.tile0[mid] <= mt_glob) lo = mid; else hi = mid;
+  }
+  r.g = lo;
+  const int mt = mt_glob - t.tile0[lo];
+  r.row0 = t.row0[lo] + (int64_t)mt * BM;
+  const int left = t.rows[lo] - mt * BM;
+  r.rows = left < BM ? left : BM;
+  r.k0 = 0;
+  r.k1 = p.K;
+  return r;
+}
+
+// Persistent walk: workgroup b of P visits tiles it*P + perm(b).  Consecutive
+// workgroup ids land on different XCDs (round robin over 8), so perm() hands
+// each XCD a contiguous run of P/8 tiles per sweep: neighbours in the tile order
+// (same expert weights, same activation rows) then share one XCD's L2.
+TGG_DEV int64_t sched_first_tile() {
+  const int P = gridDim.x, b = blockIdx.x;
+  if ((P & 7) == 0) return (int64_t)(b & 7) * (P >> 3) + (b >> 3);
+  return b;
+}
+
+}  // namespace tgg

@@ -1,0 +1,103 @@
+"""Contiguous ("DeepGEMM-style") grouped GEMM entry points, served natively.
+
+The reference's gemm/deep_gemm_ops.py:24-100 validates shapes, builds the per-row group
+layout and hands the arithmetic to the external ``deep_gemm`` package.  Here the same two
+functions, with the same signatures and ``ValueError`` checks, run this library's own gfx950
+kernels: A (and the output) are physically padded so that every expert starts at a multiple of
+``block_m`` rows; ``size_per_group`` holds the real row counts.  Rows in the padding are not
+written.
+
+``grouped_layout`` is what the reference forwards to ``deep_gemm``; it is redundant with
+``size_per_group`` and ``block_m``, so it is accepted and only shape-checked.  The psum form
+(``use_psum_layout=True``) describes the same placement and takes the same path.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from .. import _native
+from .BF16.m_grouped_gemm import _sizes_on_device
+from .layout import round_up_to_alignment
+
+
+def _check_contiguous_layout(a: torch.Tensor, b: torch.Tensor, size_per_group: torch.Tensor, block_m: int,
+                             grouped_layout: Optional[torch.Tensor], use_psum_layout: bool, what: str):
+    if a.dim() != 2 or b.dim() != 3:
+        raise ValueError(f"expected {what} shape [M, K] and b shape [num_groups, N, K]")
+    m, k = a.shape
+    g, n, bk = b.shape
+    if bk != k:
+        raise ValueError(f"K mismatch: a has K={k}, b has K={bk}")
+    if size_per_group.dim() != 1 or size_per_group.shape[0] != g:
+        raise ValueError(f"size_per_group must hold {g} entries")
+    expected_m = int(round_up_to_alignment(size_per_group.to(dtype=torch.int32), block_m).sum().item())
+    if m != expected_m:
+        raise ValueError(f"A must include padded expert rows: expected M={expected_m}, got M={m}")
+    if grouped_layout is not None:
+        want = g if use_psum_layout else m
+        if grouped_layout.dim() != 1 or grouped_layout.shape[0] != want:
+            raise ValueError(f"grouped_layout must have {want} entries")
+    return m, n, k, g
+
+
+def m_grouped_bf16_nt_contiguous(a: torch.Tensor, b: torch.Tensor, size_per_group: torch.Tensor, *,
+                                 out: Optional[torch.Tensor] = None, grouped_layout: Optional[torch.Tensor] = None,
+                                 block_m: int = 128, use_psum_layout: bool = False) -> torch.Tensor:
+    """a ``[M_padded, K]`` bf16, b ``[G, N, K]`` bf16 -> ``[M_padded, N]`` bf16
+    (reference gemm/deep_gemm_ops.py:24-57)."""
+    m, n, k, g = _check_contiguous_layout(a, b, size_per_group, block_m, grouped_layout, use_psum_layout, "a")
+    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
+        raise ValueError("a and b must be bfloat16")
+    if out is None:
+        out = torch.empty((m, n), device=a.device, dtype=torch.bfloat16)
+    _native.require_gpu(a, b, out)
+    if not (a.is_contiguous() and b.is_contiguous() and out.is_contiguous()):
+        raise ValueError("a, b and out must be contiguous")
+    sizes, is64 = _sizes_on_device(size_per_group, a.device)
+    _native.call("tgg_m_grouped_gemm_padded", a.data_ptr(), b.data_ptr(), out.data_ptr(), sizes.data_ptr(), is64, g,
+                 m, n, k, int(block_m), _native.BF16, -1, _native.stream_of(a))
+    return out
+
+
+def m_grouped_fp8_nt_contiguous(a: Tuple[torch.Tensor, torch.Tensor], b: Tuple[torch.Tensor, torch.Tensor],
+                                size_per_group: torch.Tensor, *, out: Optional[torch.Tensor] = None,
+                                grouped_layout: Optional[torch.Tensor] = None,
+                                recipe_a: Optional[Tuple[int, int]] = None,
+                                recipe_b: Optional[Tuple[int, int]] = None, block_m: int = 128,
+                                use_psum_layout: bool = False) -> torch.Tensor:
+    """Block-scaled FP8 grouped GEMM (reference gemm/deep_gemm_ops.py:60-100).
+
+    ``a = (codes [M_padded, K] e4m3fn, scales [M_padded, K/128] fp32)`` (1x128 recipe),
+    ``b = (codes [G, N, K] e4m3fn, scales [G, ceil(N/128), K/128] fp32)`` (128x128 recipe).
+    ``out[r, n] = sum_kb (sum_{k in kb} a[r,k] b[g,n,k]) * sa[r,kb] * sb[g, n//128, kb]`` with the
+    scaling applied to the fp32 accumulator once per 128-deep K block; bf16 output.
+    """
+    a_codes, a_scale = a
+    b_codes, b_scale = b
+    m, n, k, g = _check_contiguous_layout(a_codes, b_codes, size_per_group, block_m, grouped_layout,
+                                          use_psum_layout, "a[0]")
+    if recipe_a not in (None, (1, 128)) or recipe_b not in (None, (128, 128)):
+        raise ValueError("only recipe_a=(1, 128) and recipe_b=(128, 128) are implemented")
+    if a_codes.dtype != torch.float8_e4m3fn or b_codes.dtype != torch.float8_e4m3fn:
+        raise ValueError("a[0] and b[0] must be float8_e4m3fn")
+    if block_m % 128 != 0:
+        raise ValueError(f"block_m must be a multiple of 128, got {block_m}")
+    kb, nb = (k + 127) // 128, (n + 127) // 128
+    if tuple(a_scale.shape) != (m, kb):
+        raise ValueError(f"a[1] must have shape ({m}, {kb}), got {tuple(a_scale.shape)}")
+    if tuple(b_scale.shape) != (g, nb, kb):
+        raise ValueError(f"b[1] must have shape ({g}, {nb}, {kb}), got {tuple(b_scale.shape)}")
+    if out is None:
+        out = torch.empty((m, n), device=a_codes.device, dtype=torch.bfloat16)
+    _native.require_gpu(a_codes, a_scale, b_codes, b_scale, out)
+    if not (a_codes.is_contiguous() and b_codes.is_contiguous() and out.is_contiguous()):
+        raise ValueError("a[0], b[0] and out must be contiguous")
+    sa = a_scale.to(torch.float32).contiguous()
+    sb = b_scale.to(torch.float32).contiguous()
+    sizes, is64 = _sizes_on_device(size_per_group, a_codes.device)
+    _native.call("tgg_m_grouped_gemm_fp8_block", a_codes.data_ptr(), sa.data_ptr(), b_codes.data_ptr(),
+                 sb.data_ptr(), out.data_ptr(), sizes.data_ptr(), is64, g, m, n, k, int(block_m), -1,
+                 _native.stream_of(a_codes))
+    return out
