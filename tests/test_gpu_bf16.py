@@ -39,6 +39,7 @@ def test_config1_tiny_reference_case(dev, variant):
     out = m_grouped_gemm(a.to(dev), b.to(dev), sizes.to(dev), True)
     rd = check_16bit_gemm(out, gemm_ref.gmm(a, b, sizes, True), gemm_ref.gmm_fp32(a, b, sizes, True), "config1")
     print(f"config1 max-norm rdiff vs bf16 torch reference: {rd:.3e}")
+    assert rd <= 1e-3  # the stated BF16 target, max-norm, on the reference's own CPU-runnable case
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

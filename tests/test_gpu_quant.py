@@ -83,7 +83,7 @@ def test_trans_quant_roundtrip_at_larger_size(dev):
         blk = deq[:, dst:dst + s].t().cpu()
         ref = x[src:src + s].float()
         sc = scales[:, dst // 128:(dst + p) // 128].repeat_interleave(128, 0).repeat_interleave(128, 1)[:, :s].t().cpu()
-        assert bool(((blk - ref).abs() <= sc * 16.0 + 1e-12).all())  # half of the largest e4m3 step (32) times scale
+        assert bool(((blk - ref).abs() <= sc * 16.0 * 1.0001 + 1e-12).all())  # half of the largest e4m3 step (32) times scale
         assert not codes[:, dst + s:dst + p].view(torch.uint8).any()
         src += s
         dst += p

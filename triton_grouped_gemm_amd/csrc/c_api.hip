@@ -133,7 +133,7 @@ int tgg_k_grouped_gemm(const void* A, const void* B, void* C, const int32_t* sta
   if ((Mdim & 7) || (N & 7)) return set_error("Mdim and N must be multiples of 8 (16-byte rows), got %d, %d", Mdim, N);
   GemmParams p = zero_params();
   p.A = A; p.B = B; p.C = C; p.k_start = start; p.k_end = end; p.G = G;
-  p.mode = MODE_KG; p.m_total = Mdim; p.N = N; p.K = 0;
+  p.mode = MODE_KG; p.m_total = Mdim; p.k_total = Ktot; p.N = N; p.K = 0;
   p.a_sm = 1; p.a_sk = Mdim; p.b_sg = 0; p.b_sn = 1; p.b_sk = N; p.c_sg = (int64_t)Mdim * N;
   p.grid_limit = num_cu;
   return dispatch_16bit(p, dtype, 2, (hipStream_t)stream);
@@ -170,7 +170,7 @@ int tgg_k_grouped_gemm_fp8_channel(const void* x, const float* xs, const void* y
   GemmParams p = zero_params();
   p.A = x; p.B = y; p.C = out; p.sizes = tokens; p.sizes_i64 = 0; p.G = G;
   p.scale_m = xs; p.scale_n = ys; p.scale_m_sg = M;
-  p.mode = MODE_KG_COUNT; p.m_total = M; p.N = N; p.K = 0;
+  p.mode = MODE_KG_COUNT; p.m_total = M; p.k_total = Ktot; p.N = N; p.K = 0;
   p.a_sm = Ktot; p.a_sk = 1; p.b_sg = 0; p.b_sn = Ktot; p.b_sk = 1; p.c_sg = (int64_t)M * N;
   p.grid_limit = num_cu;
   return launch_generic_fp8_channel(p, fmt_a, fmt_b, TGG_BF16, (hipStream_t)stream);
@@ -197,7 +197,7 @@ int tgg_m_grouped_gemm_fp8_block(const void* Aq, const float* sa, const void* Bq
 int tgg_trans_per_block_quant_expand_128x(const void* x, void* codes, float* scales, const void* sizes,
                                           int sizes_i64, int G, int64_t M, int N, int64_t M_expand, int fmt,
                                           void* stream) {
-  if (!x || !codes || !scales || !sizes) return set_error("null pointer");
+  if ((!x && M > 0) || !codes || !scales || !sizes) return set_error("null pointer");
   if (G < 1 || G > TGG_MAX_GROUPS) return set_error("G=%d outside [1, %d]", G, TGG_MAX_GROUPS);
   if (N < 128 || (N & 127)) return set_error("N must be a positive multiple of 128, got %d", N);
   if (M < 0 || M_expand < 0 || (M_expand & 127)) return set_error("M_expand must be a multiple of 128");

@@ -71,6 +71,7 @@ struct GemmParams {
   const float* sb;        // block-scaled: [G, ceil(N/128), ceil(K/128)] weight scales
   int64_t m_total;        // rows of A/C that may be touched (M-grouped), Mdim for K-grouped
   int64_t m_stride;       // MODE_MASKED: rows between consecutive groups
+  int64_t k_total;        // K-grouped: length of the shared reduction axis (segments are clipped to it)
   int64_t a_sm, a_sk;
   int64_t b_sg, b_sn, b_sk;
   int64_t c_sg;           // K-grouped: elements between consecutive groups' outputs

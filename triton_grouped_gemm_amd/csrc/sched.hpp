@@ -38,6 +38,8 @@ TGG_DEV void sched_init(const GemmParams& p, SchedTable& t) {
   if (p.mode == MODE_KG) {
     for (int g = threadIdx.x; g < G; g += blockDim.x) {
       int64_t s = p.k_start[g], e = p.k_end[g];
+      if (s < 0) s = 0;
+      if (e > p.k_total) e = p.k_total;
       t.row0[g] = s;
       t.rows[g] = e > s ? (int32_t)(e - s) : 0;
     }
@@ -59,10 +61,9 @@ TGG_DEV void sched_init(const GemmParams& p, SchedTable& t) {
         start = row;
         row += (p.mode == MODE_MG_PAD) ? ((sz + p.align - 1) / p.align) * p.align : sz;
       }
-      if (p.mode != MODE_KG_COUNT) {  // never touch rows past the end of A / C
-        if (start >= p.m_total) sz = 0;
-        else if (start + sz > p.m_total) sz = p.m_total - start;
-      }
+      const int64_t limit = (p.mode == MODE_KG_COUNT) ? p.k_total : p.m_total;
+      if (start >= limit) sz = 0;  // never touch rows (or k) past the end of the operands
+      else if (start + sz > limit) sz = limit - start;
       t.row0[g] = start;
       t.rows[g] = (int32_t)sz;
       t.tile0[g] = tile;
