@@ -1,0 +1,194 @@
+#!/usr/bin/env python3
+"""Headline benchmark: BF16 M-grouped GEMM, G=128, M=655360, N=1536, K=2048 on one MI355X.
+
+One "step" is one pass of the hot path (one ``m_grouped_gemm`` launch) over a synthetic batch whose
+operands are already resident in HBM.  Prints ONE JSON line: TFLOP/s = 2*M*N*K / time, the MFMA
+roofline fraction of the GEMM kernel (HIP-event timed on the launch stream) and, beside it, the
+reference's per-group torch matmul timed on this box's host cores over a bounded sample of groups.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0}   # MI355X dense MFMA peaks
+PEAK_HBM_GBS = 8000.0
+
+G, M_TOTAL = 128, 655360
+WORKLOADS = {
+    # name: (kind, N, K, trans_b)
+    "bf16_m_grouped_gateup_nt": ("mg", 1536, 2048, True),
+    "bf16_m_grouped_gateup_nn": ("mg", 1536, 2048, False),
+    "bf16_m_grouped_down_nt": ("mg", 2048, 768, True),
+    "bf16_m_grouped_down_nn": ("mg", 2048, 768, False),
+    "bf16_masked_decode": ("masked", 4096, 1536, True),
+    "bf16_k_grouped_wgrad": ("kg", 4096, 3072, False),      # N_DIM, M_DIM
+    "fp8_block_m_grouped": ("fp8", 3072, 4096, True),
+    "quant_trans128": ("quant", 4096, 0, False),
+}
+
+
+def build_workload(name: str, dev, seed: int = 2026):
+    """Returns (fn, flops_per_step, algorithmic_bytes_per_step, dtype_tag, description, cpu_sample_fn)."""
+    from triton_grouped_gemm_amd import workloads as wl
+    from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm_TMA import m_grouped_gemm
+    kind, N, K, trans_b = WORKLOADS[name]
+    sizes_cpu = wl.dirichlet_multinomial_sizes(G, M_TOTAL, 128, seed=seed)
+    sizes = sizes_cpu.to(dev)
+    if kind == "mg":
+        a = wl.randn_bf16((M_TOTAL, K), K ** -0.5, seed + 1, dev)
+        b = wl.randn_bf16((G, N, K) if trans_b else (G, K, N), K ** -0.5, seed + 2, dev)
+        fn = lambda: m_grouped_gemm(a, b, sizes, trans_b)
+        flops = 2.0 * M_TOTAL * N * K
+        nbytes = 2.0 * M_TOTAL * K + 2.0 * G * N * K + 2.0 * M_TOTAL * N
+
+        def cpu_sample(budget_s: float):
+            from oracle import gemm_ref
+            order = torch.argsort(sizes_cpu, descending=True).tolist()
+            starts = (sizes_cpu.cumsum(0) - sizes_cpu).tolist()
+            done_flops, t_used, groups = 0.0, 0.0, 0
+            warm = True
+            for g in order:
+                n = int(sizes_cpu[g])
+                if n == 0:
+                    continue
+                ag = a[starts[g]:starts[g] + n].cpu()
+                bg = b[g:g + 1].cpu()
+                if warm:
+                    gemm_ref.gmm(ag[:256], bg, [256], trans_b)
+                    warm = False
+                t0 = time.perf_counter()
+                gemm_ref.gmm(ag, bg, [n], trans_b)
+                t_used += time.perf_counter() - t0
+                done_flops += 2.0 * n * N * K
+                groups += 1
+                if t_used >= budget_s:
+                    break
+            return done_flops / t_used / 1e12, f"{groups} largest groups of {G} ({done_flops / flops * 100:.1f}% of the step's flops), bf16 torch matmul per group"
+        return fn, flops, nbytes, "bf16", dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, trans_b=trans_b,
+                                               group_sizes="dirichlet-multinomial, 128-aligned", seed=seed), cpu_sample
+    if kind == "masked":
+        from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm_masked_TMA import m_grouped_gemm_masked
+        m_max = 512
+        mm_cpu = wl.masked_counts(G, m_max, seed)
+        mm = mm_cpu.to(dev)
+        lhs = wl.randn_bf16((G * m_max, K), K ** -0.5, seed + 1, dev)
+        rhs = wl.randn_bf16((G, N, K), K ** -0.5, seed + 2, dev)
+        out = torch.empty((G * m_max, N), device=dev, dtype=torch.bfloat16)
+        mv = float(mm_cpu.sum())
+        fn = lambda: m_grouped_gemm_masked(lhs, rhs, out, mm, m_max)
+        return (fn, 2.0 * mv * N * K, 2.0 * mv * K + 2.0 * int((mm_cpu > 0).sum()) * N * K + 2.0 * mv * N, "bf16",
+                dict(workload=name, G=G, m_max=m_max, N=N, K=K, valid_rows=int(mv), seed=seed), None)
+    if kind == "kg":
+        from triton_grouped_gemm_amd.gemm.BF16.k_grouped_gemm_TMA import k_grouped_gemm
+        Nd, Md = N, K
+        a = wl.randn_bf16((M_TOTAL, Md), 1.0, seed + 1, dev)
+        b = wl.randn_bf16((M_TOTAL, Nd), 1.0, seed + 2, dev)
+        fn = lambda: k_grouped_gemm(a, b, sizes)
+        return (fn, 2.0 * M_TOTAL * Md * Nd, 2.0 * M_TOTAL * (Md + Nd) + 2.0 * G * Md * Nd, "bf16",
+                dict(workload=name, G=G, K_total=M_TOTAL, M_dim=Md, N_dim=Nd, seed=seed), None)
+    if kind == "fp8":
+        from triton_grouped_gemm_amd.gemm.deep_gemm_ops import m_grouped_fp8_nt_contiguous
+        from triton_grouped_gemm_amd.quant.fp8_cast import per_block_cast_to_fp8, per_token_cast_to_fp8
+        a = wl.randn_bf16((M_TOTAL, K), 1.0, seed + 1, dev)
+        aq = per_token_cast_to_fp8(a)
+        del a
+        w = wl.randn_bf16((G, N, K), 1.0, seed + 2, dev)
+        wq = per_block_cast_to_fp8(w)
+        del w
+        out = torch.empty((M_TOTAL, N), device=dev, dtype=torch.bfloat16)
+        fn = lambda: m_grouped_fp8_nt_contiguous(aq, wq, sizes, out=out)
+        nbytes = M_TOTAL * K + 4.0 * M_TOTAL * K / 128 + G * N * K + 4.0 * G * (N / 128) * (K / 128) + 2.0 * M_TOTAL * N
+        return (fn, 2.0 * M_TOTAL * N * K, nbytes, "fp8",
+                dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, recipe="1x128 act / 128x128 weight, e4m3fn", seed=seed), None)
+    if kind == "quant":
+        from triton_grouped_gemm_amd.quant.trans_per_block_quant_expand_128x import trans_per_block_quant_expand_128x
+        x = wl.randn_bf16((M_TOTAL, N), 1.0, seed + 1, dev)
+        me = M_TOTAL + 128 * G - M_TOTAL % 128
+        fn = lambda: trans_per_block_quant_expand_128x(x, sizes)
+        nbytes = 2.0 * M_TOTAL * N + 1.0 * N * me + 4.0 * (N / 128) * (me / 128)
+        return fn, 0.0, nbytes, "bf16->fp8", dict(workload=name, G=G, M=M_TOTAL, N=N, seed=seed), None
+    raise ValueError(name)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="bf16_m_grouped_gateup_nt", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="host-core time budget of the CPU baseline sample")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: the grouped-GEMM path has no cross-GPU step; run with --gpus 1", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (there is no CPU path)", file=sys.stderr)
+        return 2
+    from triton_grouped_gemm_amd import _native
+    _native.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    fn, flops, nbytes, dtype_tag, config, cpu_sample = build_workload(args.workload, dev)
+
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream(dev)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for s, e in evs:
+        s.record(stream)
+        fn()
+        e.record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kernel_ms = [s.elapsed_time(e) for s, e in evs]
+    avg_kernel_ms = sum(kernel_ms) / len(kernel_ms)
+
+    is_gemm = flops > 0
+    if is_gemm:
+        value = flops / (wall_ms * 1e-3) / 1e12
+        peak = PEAK_TFLOPS["fp8" if dtype_tag == "fp8" else "bf16"]
+        achieved = flops / (avg_kernel_ms * 1e-3) / 1e12
+        roofline = dict(bound="mfma", achieved=round(achieved, 2), peak=peak, unit="TFLOP/s",
+                        frac=round(achieved / peak, 4), traffic=None,
+                        min_ms=round(min(kernel_ms), 4), avg_ms=round(avg_kernel_ms, 4),
+                        algorithmic_gbytes=round(nbytes / 1e9, 3))
+        metric, unit = "grouped GEMM TFLOP/s (2*M*N*K/time), M-grouped G=128", "TFLOP/s"
+    else:
+        value = nbytes / (wall_ms * 1e-3) / 1e9
+        achieved = nbytes / (avg_kernel_ms * 1e-3) / 1e9
+        roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                        frac=round(achieved / PEAK_HBM_GBS, 4), traffic=None,
+                        min_ms=round(min(kernel_ms), 4), avg_ms=round(avg_kernel_ms, 4))
+        metric, unit = "quantizer algorithmic GB/s", "GB/s"
+
+    cpu_baseline = None
+    if cpu_sample is not None and not args.no_cpu_baseline:
+        tf, sample = cpu_sample(args.cpu_seconds)
+        cpu_baseline = dict(value=round(tf, 4), unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                            sample=sample, host_cpus=os.cpu_count())
+
+    print(json.dumps({
+        "metric": metric, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": dtype_tag, "data": "synthetic", "config": config,
+        "roofline": roofline, "cpu_baseline": cpu_baseline,
+    }))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

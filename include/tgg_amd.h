@@ -94,7 +94,8 @@ int tgg_per_block_cast_to_fp8(const void* x, void* codes, float* scales, int bat
  * `.to(torch.float8_*)` casts of the recipes above). */
 int tgg_cvt_f32_to_fp8(const float* in, void* out, int64_t n, int fmt, void* stream);
 
-/* Library controls: "force_generic" (0/1) routes every GEMM through the shape-agnostic kernel. */
+/* Library controls: "force_generic" (0/1) routes every GEMM through the shape-agnostic kernel;
+ * "variant" (int) selects a tile configuration of the tuned kernels (0 = default). */
 int tgg_set_option(const char* key, int value);
 const char* tgg_last_error(void);
 int tgg_version(void);

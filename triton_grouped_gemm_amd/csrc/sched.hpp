@@ -11,11 +11,14 @@ namespace tgg {
 
 constexpr int kMaxGroups = 1024;
 
-struct SchedTable {
-  int64_t row0[kMaxGroups];     // first row of the group in A/C (M modes) or first k (K modes)
-  int32_t rows[kMaxGroups];     // valid rows (M modes) or k extent (K modes)
-  int32_t tile0[kMaxGroups + 1];// exclusive prefix of ceil(rows / BM) (M modes only)
+template <int MAXG>
+struct SchedTableT {
+  int64_t row0[MAXG];      // first row of the group in A/C (M modes) or first k (K modes)
+  int32_t rows[MAXG];      // valid rows (M modes) or k extent (K modes)
+  int32_t tile0[MAXG + 1]; // exclusive prefix of ceil(rows / BM) (M modes only)
+  int32_t pad_;
 };
+typedef SchedTableT<kMaxGroups> SchedTable;
 
 struct Tile {
   int g;
@@ -32,8 +35,8 @@ TGG_DEV int64_t load_size(const void* p, int is64, int i) {
 }
 
 // All threads of the workgroup must call this; ends with a barrier.
-template <int BM>
-TGG_DEV void sched_init(const GemmParams& p, SchedTable& t) {
+template <int BM, class Table>
+TGG_DEV void sched_init(const GemmParams& p, Table& t) {
   const int G = p.G;
   if (p.mode == MODE_KG) {
     for (int g = threadIdx.x; g < G; g += blockDim.x) {
@@ -74,8 +77,8 @@ TGG_DEV void sched_init(const GemmParams& p, SchedTable& t) {
   __syncthreads();
 }
 
-template <int BM, int BN>
-TGG_DEV int64_t sched_num_tiles(const GemmParams& p, const SchedTable& t) {
+template <int BM, int BN, class Table>
+TGG_DEV int64_t sched_num_tiles(const GemmParams& p, const Table& t) {
   const int tiles_n = (p.N + BN - 1) / BN;
   if (p.mode == MODE_KG || p.mode == MODE_KG_COUNT) {
     const int tiles_m = (int)((p.m_total + BM - 1) / BM);
@@ -84,8 +87,8 @@ TGG_DEV int64_t sched_num_tiles(const GemmParams& p, const SchedTable& t) {
   return (int64_t)t.tile0[p.G] * tiles_n;
 }
 
-template <int BM, int BN>
-TGG_DEV Tile sched_tile(const GemmParams& p, const SchedTable& t, int64_t tile_id) {
+template <int BM, int BN, class Table>
+TGG_DEV Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id) {
   Tile r;
   const int tiles_n = (p.N + BN - 1) / BN;
   if (p.mode == MODE_KG || p.mode == MODE_KG_COUNT) {
