@@ -46,6 +46,7 @@ int launch_cvt_fp8(const float*, void*, int64_t, int, hipStream_t);
 bool fast_supported(const GemmParams& p, int dt, int layout);
 int launch_fast_16bit(const GemmParams& p, int dt, int layout, hipStream_t s);
 void set_fast_variant(int v);
+void set_tile_order(int v);
 
 static bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 
@@ -233,6 +234,7 @@ int tgg_cvt_f32_to_fp8(const float* in, void* out, int64_t n, int fmt, void* str
 int tgg_set_option(const char* key, int value) {
   if (key && strcmp(key, "force_generic") == 0) { g_force_generic = value != 0; return 0; }
   if (key && strcmp(key, "variant") == 0) { set_fast_variant(value); return 0; }
+  if (key && strcmp(key, "tile_order") == 0) { set_tile_order(value); return 0; }
   return set_error("unknown option '%s'", key ? key : "(null)");
 }
 

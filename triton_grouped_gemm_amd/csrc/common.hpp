@@ -83,6 +83,7 @@ struct GemmParams {
   int N;
   int K;                  // reduction length (M-grouped); unused for K-grouped
   int grid_limit;         // >0 caps the persistent grid
+  int tile_order;         // 0: XCD-contiguous tile runs, 1: plain round robin
 };
 
 }  // namespace tgg
