@@ -1,16 +1,26 @@
-// Tuned bf16/fp16 grouped GEMM for gfx950, K-contiguous operands ("NT": A [rows, K], B [G, N, K]).
+// Tuned bf16/fp16 grouped GEMM kernels for gfx950.
 //
-// Persistent workgroups walk the grouped tile space (sched.hpp).  Per tile:
-//   * A and B slabs of BK columns stream HBM/L2 -> LDS with buffer_load_dwordx4 ... lds
-//     (no VGPR staging); rows past the end of the operand read as zero through the buffer
-//     descriptor's bounds check, so ragged groups need no special path;
-//   * NSTAGE slabs are in flight; one barrier per slab;
-//   * LDS rows are XOR-swizzled at 16-byte granularity (applied on the global side of the
-//     direct-to-LDS copy, whose LDS side is lane-linear) so that ds_read_b128 fragment reads
-//     are bank-conflict free;
-//   * each wave owns a (BM/WM) x (BN/WN) block of 32x32x16 MFMA tiles, issued with the
-//     weights as srcA and the activations as srcB so a lane ends up with 4 consecutive
-//     output columns of one row.
+// One kernel template covers the three operand layouts of the grouped-GEMM path:
+//   NT  A [rows, K]      B [G, N, K]   (forward, masked/decode, contiguous-padded)
+//   NN  A [rows, K]      B [G, K, N]   (activation gradient)
+//   TN  A [Ktot, Mdim]   B [Ktot, N]   (K-grouped weight gradient, per-group token range)
+//
+// Persistent workgroups walk the grouped tile space (sched.hpp).  Per 256x256 (or smaller) tile:
+//   * 64-deep K slabs of both operands stream HBM/L2 -> LDS with buffer_load_dwordx4 ... lds, no
+//     VGPR staging.  Anything outside an operand (rows past the end of A, tokens past the end of
+//     a group's range) reads as zero through the buffer descriptor's bounds check, so ragged
+//     groups and token tails need no separate code path.
+//   * NSTAGE slabs rotate through LDS with one workgroup barrier per slab; the first slabs of the
+//     next tile are requested before the current tile's results are drained.
+//   * LDS is XOR-swizzled at 16-byte granularity.  The direct-to-LDS copy is lane-linear on the
+//     LDS side, so the swizzle is applied to the global address each lane fetches from.
+//   * K-contiguous operands are read back as 16-byte MFMA fragments (ds_read_b128); operands whose
+//     rows are tokens (MN-contiguous) are read with the transposing ds_read_b64_tr_b16, which hands
+//     every lane 4 consecutive K values of one column.
+//   * Each wave owns a (BM/WM) x (BN/WN) block of 32x32x16 MFMA tiles, issued with the B operand as
+//     srcA and the A operand as srcB, so a lane ends up with 4 consecutive output columns of one
+//     row; results are transposed through a per-wave LDS staging area and leave as 16-byte stores
+//     covering whole 128-byte row segments.
 #include "common.hpp"
 #include "sched.hpp"
 #include "launch.hpp"
@@ -20,6 +30,9 @@ namespace tgg {
 namespace {
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __attribute__((address_space(3))) i16x4_t* lds_i16x4_ptr_t;
+
+enum : int { LAYOUT_NT = 0, LAYOUT_NN = 1, LAYOUT_TN = 2 };
 
 template <int DT> struct Mma16;
 template <> struct Mma16<DT_BF16> {
@@ -48,58 +61,78 @@ TGG_DEV void copy_b128_to_lds(i32x4_t rsrc, uint32_t lds_addr, int voff) {
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
 }
 
-// Same, 4 bytes per lane (LDS destination m0 + lane * 4).
-TGG_DEV void copy_b32_to_lds(i32x4_t rsrc, uint32_t lds_addr, int voff) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
-}
+// A run of slabs of one operand: slab kt starts at base + kt * step and may touch `bytes - kt * step`
+// bytes from there (everything beyond reads as zero).  All fields are wave-uniform.
+struct Stream {
+  uint64_t base;
+  int64_t bytes;
+  int64_t step;
+};
 
-TGG_DEV i32x4_t make_rsrc(const void* base, uint32_t num_bytes) {
-  const uint64_t a = (uint64_t)base;
-  i32x4_t r;  // wave-uniform by construction; readfirstlane pins it to scalar registers
+TGG_DEV i32x4_t stream_rsrc(const Stream& s, int kt) {
+  const uint64_t a = s.base + (uint64_t)(kt * s.step);
+  int64_t left = s.bytes - kt * s.step;
+  left = left < 0 ? 0 : (left > 0x7fffffff ? 0x7fffffff : left);
+  i32x4_t r;  // readfirstlane pins the descriptor to scalar registers
   r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
   r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32) & 0xffff);  // stride 0, no swizzle
-  r[2] = __builtin_amdgcn_readfirstlane((int)num_bytes);
-  r[3] = 0x00020000;                                                          // raw 32-bit data format
+  r[2] = __builtin_amdgcn_readfirstlane((int)left);
+  r[3] = 0x00020000;  // raw buffer, 32-bit data format
   return r;
 }
 
 constexpr int kFastMaxGroups = 256;
+constexpr int BK = 64;  // K depth of a slab: 128 bytes of a K-contiguous row
 
-// PFD: how many slabs beyond the one being copied the L2 warm-up reads run (0 = no warm-up).
-template <int BM_, int BN_, int BK_, int NSTAGE_, int WM_, int WN_, int PFD_ = 2>
-struct FastCfg {
-  static constexpr int BM = BM_, BN = BN_, BK = BK_, NSTAGE = NSTAGE_, WM = WM_, WN = WN_, PFD = PFD_;
-  static constexpr int NWAVES = WM * WN;
-  static constexpr int THREADS = NWAVES * 64;
-  static constexpr int RB = BK * 2;            // bytes per LDS row
-  static constexpr int CPR = RB / 16;          // 16-byte chunks per row
-  static constexpr int RPB = 256 / RB;         // rows per 256 bytes (one pass over all banks)
-  static constexpr int RPI = 1024 / RB;        // rows written by one wave-wide direct-to-LDS load
-  static constexpr int NI_A = BM / RPI, NI_B = BN / RPI;   // load instructions per slab
-  static constexpr int NI = NI_A + NI_B;
-  static constexpr int NCOPY = PFD > 0 ? NWAVES / 2 : NWAVES;  // waves that issue the slab copies
-  static constexpr int NTOUCH = NWAVES - NCOPY;                // waves that issue L2 warm-up reads instead
-  static constexpr int LPW = NI / NCOPY;       // copies per copying wave per slab
-  static constexpr int A_BYTES = BM * RB, B_BYTES = BN * RB;
-  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-  static constexpr int NPAT = (RPB * CPR) / RPI > 1 ? (RPB * CPR) / RPI : 1;  // distinct swizzle patterns over load instrs
-  static constexpr int EPI_PITCH = (BN / WN) * 2 + 16;   // staged output row pitch in bytes
-  static constexpr int EPI_WAVE_BYTES = 32 * EPI_PITCH;
-  static constexpr int PFW = PFD > 0 ? ((BM + BN) / 64 + NTOUCH - 1) / NTOUCH : 0;  // warm-up reads per touching wave per slab
-  static constexpr int SINK_OFFSET = NSTAGE * STAGE_BYTES + (int)sizeof(SchedTableT<kFastMaxGroups>);
-  static constexpr int SMEM_BYTES = SINK_OFFSET + NWAVES * 256;
-  static_assert(BM % 64 == 0 && BN % 64 == 0, "warm-up split");
-  static_assert(PFD == 0 || BK == 64, "warm-up reads assume one 128-byte line per slab row");
-  static_assert(NWAVES * EPI_WAVE_BYTES <= STAGE_BYTES, "epilogue staging must fit in one slab buffer");
-  static_assert(NI_A % NCOPY == 0 && NI_B % NCOPY == 0, "copies must divide evenly over the copying waves");
-  static_assert(LPW * (NSTAGE - 1) < 64, "vmcnt range");
+// Geometry of one operand's slab in LDS and of the copies that fill it.
+//   KMAJOR: ROWS rows of 128 bytes (64 K values each).  A copy instruction covers 8 rows; the
+//           16-byte chunk c of row r sits at slot c ^ ((r / 2) % 8).
+//   !KMAJOR: 64 token rows of ROWS*2 bytes.  A copy instruction covers 1024 / (ROWS*2) token rows;
+//           chunk c of token row k sits at slot c ^ ((k % 4) * 4).
+template <int ROWS, bool KMAJOR> struct Operand {
+  static constexpr int SLAB_BYTES = ROWS * BK * 2;
+  static constexpr int NI = SLAB_BYTES / 1024;                 // copy instructions per slab
+  static constexpr int ROW_BYTES = KMAJOR ? BK * 2 : ROWS * 2; // bytes of one LDS row
+  static constexpr int CPR = ROW_BYTES / 16;                   // 16-byte chunks per LDS row
+  static constexpr int RPI = 1024 / ROW_BYTES;                 // LDS rows per copy instruction
+  static constexpr int NPAT = KMAJOR ? 2 : (RPI >= 4 ? 1 : 4 / RPI);  // swizzle patterns over instructions
+
+  // byte offset (from the slab's first byte in global memory) fetched by `lane` of a copy
+  // instruction with swizzle pattern `pat`; ld = bytes between consecutive global rows.
+  static TGG_DEV int lane_voff(int lane, int pat, int ld) {
+    const int r_local = lane / CPR, slot = lane % CPR;
+    const int r = pat * RPI + r_local;  // row index modulo the swizzle period
+    const int sw = KMAJOR ? (r / 2) % 8 : (r % 4) * 4;
+    return r_local * ld + ((slot ^ sw) << 4);
+  }
 };
 
-// DBG is a development aid for isolating pipeline stages: bit 0 drops the slab copies, bit 1 the
-// fragment reads, bit 2 the MFMAs (results are then meaningless).
-template <class C, int DT, int DBG = 0>
-__global__ __launch_bounds__(C::THREADS) void gemm_fast_nt_kernel(const GemmParams p) {
+template <int BM_, int BN_, int NSTAGE_, int WM_, int WN_>
+struct FastCfg {
+  static constexpr int BM = BM_, BN = BN_, NSTAGE = NSTAGE_, WM = WM_, WN = WN_;
+  static constexpr int NWAVES = WM * WN;
+  static constexpr int THREADS = NWAVES * 64;
+  static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int NI_A = A_BYTES / 1024, NI_B = B_BYTES / 1024;
+  static constexpr int LPW = (NI_A + NI_B) / NWAVES;  // copies per wave per slab
+  static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+  static constexpr int EPI_PITCH = (BN / WN) * 2 + 16;  // staged output row pitch in bytes
+  static constexpr int EPI_WAVE_BYTES = 32 * EPI_PITCH;
+  static constexpr int SMEM_BYTES = NSTAGE * STAGE_BYTES + (int)sizeof(SchedTableT<kFastMaxGroups>);
+  static_assert(NI_A % NWAVES == 0 && NI_B % NWAVES == 0, "copies must divide evenly over waves");
+  static_assert(NWAVES % 4 == 0, "a wave keeps one swizzle pattern for all its copies");
+  static_assert(LPW * (NSTAGE - 1) < 64, "vmcnt range");
+  static_assert(NWAVES * EPI_WAVE_BYTES <= STAGE_BYTES, "epilogue staging must fit in one slab buffer");
+};
+
+template <class C, int DT, int LAYOUT>
+__global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams p) {
+  constexpr bool A_KMAJOR = LAYOUT != LAYOUT_TN;
+  constexpr bool B_KMAJOR = LAYOUT == LAYOUT_NT;
+  typedef Operand<C::BM, A_KMAJOR> OpA;
+  typedef Operand<C::BN, B_KMAJOR> OpB;
+
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::NSTAGE * C::STAGE_BYTES);
   sched_init<C::BM>(p, sched);
@@ -111,110 +144,109 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_nt_kernel(const GemmPara
   const int wm0 = (wave / C::WN) * (C::BM / C::WM);
   const int wn0 = (wave % C::WN) * (C::BN / C::WN);
   const int l32 = lane & 31, lh = lane >> 5;
-  const int K = p.K;
-  const int kt_n = K / C::BK;
-  const int row_bytes = K * 2;
 
-  // Per-lane byte offset of a direct-to-LDS load relative to (first row of the instruction, k = 0):
-  // lane -> (row l / CPR, LDS slot l % CPR); the slot holds logical chunk slot ^ f(row).
-  int ld_voff[C::NPAT];
+  // global row pitches in bytes
+  const int64_t a_ld = (LAYOUT == LAYOUT_TN ? p.m_total : (int64_t)p.K) * 2;
+  const int64_t b_ld = (LAYOUT == LAYOUT_NT ? (int64_t)p.K : (int64_t)p.N) * 2;
+
+  // per-lane source offsets of this wave's copies (one swizzle pattern per wave, see FastCfg)
+  const int a_voff = OpA::lane_voff(lane, wave % OpA::NPAT, (int)a_ld);
+  const int b_voff = OpB::lane_voff(lane, wave % OpB::NPAT, (int)b_ld);
+
+  // per-lane LDS offsets of the fragment reads, relative to the operand's slab
+  //   K-contiguous: 16 bytes = K values 16 ks + 8 lh + (0..7) of row (block + l32)
+  //   token rows:   lane L of a 16-lane group loads 8 bytes of token row (L % 16) / 4; the transposing
+  //                 read returns to lane i the 4 tokens of column i of the group
+  int a_rd[A_KMAJOR ? BK / 16 : C::TM];
+  int b_rd[B_KMAJOR ? BK / 16 : C::TN];
+  if (A_KMAJOR) {
 #pragma unroll
-  for (int pt = 0; pt < C::NPAT; ++pt) {
-    const int r = pt * C::RPI + lane / C::CPR;
-    const int f = (r / C::RPB) % C::CPR;
-    ld_voff[pt] = (lane / C::CPR) * row_bytes + (((lane % C::CPR) ^ f) << 4);
+    for (int ks = 0; ks < BK / 16; ++ks) a_rd[ks] = (wm0 + l32) * 128 + (((2 * ks + lh) ^ ((l32 / 2) % 8)) << 4);
+  } else {
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i) {
+      const int blk = lane >> 4, j = lane & 15, e = j >> 2, c = j & 3;
+      const int chunk = ((wm0 + 32 * i) / 8 + (blk & 1) * 2 + (c >> 1)) ^ (e * 4);
+      a_rd[i] = ((blk >> 1) * 8 + e) * (C::BM * 2) + chunk * 16 + (c & 1) * 8;
+    }
   }
-  static_assert(C::NCOPY % C::NPAT == 0, "static load split");
-  // With warm-up enabled the waves split roles for memory traffic (all of them compute): the lower
-  // half issues every slab copy, the upper half only issues warm-up reads.  vmcnt retires in
-  // order, so a wave that mixed both would have its copies' completion held up by the slow,
-  // far-ahead warm-up reads; a touching wave never waits on vmcnt at all.
-  const bool copier = wave < C::NCOPY;
-  const int my_voff = ld_voff[wave % C::NPAT];  // every copy of this wave uses the same swizzle pattern
-  // Per-lane LDS byte offsets of the fragment reads, relative to the operand's slab base.
-  const int fsw = (l32 / C::RPB) % C::CPR;
-  int rd_off[C::BK / 16];
+  if (B_KMAJOR) {
 #pragma unroll
-  for (int ks = 0; ks < C::BK / 16; ++ks) rd_off[ks] = l32 * C::RB + (((2 * ks + lh) ^ fsw) << 4);
+    for (int ks = 0; ks < BK / 16; ++ks) b_rd[ks] = (wn0 + l32) * 128 + (((2 * ks + lh) ^ ((l32 / 2) % 8)) << 4);
+  } else {
+#pragma unroll
+    for (int j2 = 0; j2 < C::TN; ++j2) {
+      const int blk = lane >> 4, j = lane & 15, e = j >> 2, c = j & 3;
+      const int chunk = ((wn0 + 32 * j2) / 8 + (blk & 1) * 2 + (c >> 1)) ^ (e * 4);
+      b_rd[j2] = ((blk >> 1) * 8 + e) * (C::BN * 2) + chunk * 16 + (c & 1) * 8;
+    }
+  }
 
-  // Buffer descriptors of a tile's A rows and B rows (pinned to scalar registers).
-  struct Desc { i32x4_t a, b; };
-  auto make_desc = [&](const Tile& t) {
-    const int64_t a_rows_left = p.m_total - t.row0;
-    const int a_rows = a_rows_left < C::BM ? (int)a_rows_left : C::BM;
-    const int b_rows = (p.N - t.n0) < C::BN ? (p.N - t.n0) : C::BN;
-    Desc d;
-    d.a = make_rsrc((const char*)p.A + t.row0 * (int64_t)row_bytes, (uint32_t)(a_rows * row_bytes));
-    d.b = make_rsrc((const char*)p.B + ((int64_t)t.g * p.N + t.n0) * (int64_t)row_bytes, (uint32_t)(b_rows * row_bytes));
-    return d;
+  struct TileIo { Stream a, b; int kt_n; };
+  auto make_io = [&](const Tile& t) {
+    TileIo io;
+    if (LAYOUT == LAYOUT_TN) {
+      const int64_t klen = t.k1 - t.k0;
+      io.kt_n = (int)((klen + BK - 1) / BK);
+      io.a.base = (uint64_t)p.A + (uint64_t)(t.k0 * a_ld + t.row0 * 2);
+      io.a.bytes = klen * a_ld - t.row0 * 2;
+      io.a.step = BK * a_ld;
+      io.b.base = (uint64_t)p.B + (uint64_t)(t.k0 * b_ld + (int64_t)t.n0 * 2);
+      io.b.bytes = klen * b_ld - (int64_t)t.n0 * 2;
+      io.b.step = BK * b_ld;
+    } else {
+      io.kt_n = p.K / BK;
+      const int64_t rows_left = p.m_total - t.row0;
+      io.a.base = (uint64_t)p.A + (uint64_t)(t.row0 * a_ld);
+      io.a.bytes = (rows_left < C::BM ? rows_left : C::BM) * a_ld;
+      io.a.step = BK * 2;
+      if (LAYOUT == LAYOUT_NT) {
+        const int n_left = p.N - t.n0;
+        io.b.base = (uint64_t)p.B + (uint64_t)(((int64_t)t.g * p.N + t.n0) * b_ld);
+        io.b.bytes = (int64_t)(n_left < C::BN ? n_left : C::BN) * b_ld;
+        io.b.step = BK * 2;
+      } else {
+        io.b.base = (uint64_t)p.B + (uint64_t)((int64_t)t.g * p.K * b_ld + (int64_t)t.n0 * 2);
+        io.b.bytes = (int64_t)p.K * b_ld - (int64_t)t.n0 * 2;
+        io.b.step = BK * b_ld;
+      }
+    }
+    return io;
   };
   // Offsets at or past this marker are outside every descriptor: such a copy fetches nothing (zeros
-  // land in LDS that nobody reads) but still occupies its slot in the vmcnt bookkeeping.
+  // land in LDS that nobody reads) but still takes its slot in the vmcnt bookkeeping.
   constexpr int kNoFetch = 0x40000000;
-  auto issue_slab = [&](const Desc& d, int kt, int buf) {
+  auto issue_slab = [&](const TileIo& io, int kt, int buf) {
     const uint32_t base = smem_addr + buf * C::STAGE_BYTES;
-    const int koff = kt < kt_n ? kt * (C::BK * 2) : kNoFetch;
-    if ((DBG & 1) || !copier) return;
+    const int ktc = kt < io.kt_n ? kt : 0;
+    const int dead = kt < io.kt_n ? 0 : kNoFetch;
+    const i32x4_t ra = stream_rsrc(io.a, ktc), rb = stream_rsrc(io.b, ktc);
 #pragma unroll
-    for (int j = 0; j < C::NI_A / C::NCOPY; ++j) {
-      const int idx = wave + j * C::NCOPY;  // wave-uniform
-      copy_b128_to_lds(d.a, base + idx * 1024, my_voff + idx * C::RPI * row_bytes + koff);
+    for (int j = 0; j < C::NI_A / C::NWAVES; ++j) {
+      const int idx = wave + j * C::NWAVES;  // wave-uniform
+      copy_b128_to_lds(ra, base + idx * 1024, a_voff + idx * OpA::RPI * (int)a_ld + dead);
     }
 #pragma unroll
-    for (int j = 0; j < C::NI_B / C::NCOPY; ++j) {
-      const int idx = wave + j * C::NCOPY;
-      copy_b128_to_lds(d.b, base + C::A_BYTES + idx * 1024, my_voff + idx * C::RPI * row_bytes + koff);
+    for (int j = 0; j < C::NI_B / C::NWAVES; ++j) {
+      const int idx = wave + j * C::NWAVES;
+      copy_b128_to_lds(rb, base + C::A_BYTES + idx * 1024, b_voff + idx * OpB::RPI * (int)b_ld + dead);
     }
-  };
-  // L2 warm-up of a slab that will be copied a few iterations from now: one 4-byte read per
-  // 128-byte line (every row of the slab is one line), dropped into a scratch corner of LDS.  The
-  // slab copies then hit in L2 instead of waiting on HBM / Infinity Cache inside the barrier.
-  const uint32_t sink_addr = smem_addr + C::SINK_OFFSET + wave * 256;
-  auto touch_slab = [&](const Desc& d, int kt) {
-    if (C::PFD == 0 || (DBG & 1) || copier) return;
-    if (kt >= kt_n) return;
-    const int koff = kt * (C::BK * 2);
-#pragma unroll
-    for (int j = 0; j < C::PFW; ++j) {
-      const int blk = (wave - C::NCOPY) + j * C::NTOUCH;  // 64-row block of the (A rows, then B rows) list
-      const bool is_a = blk * 64 < C::BM;            // wave-uniform
-      const int row = blk * 64 - (is_a ? 0 : C::BM) + lane;
-      if (blk * 64 < C::BM + C::BN) copy_b32_to_lds(is_a ? d.a : d.b, sink_addr, row * row_bytes + koff);
-    }
-  };
-  // Slab `s` counted from the start of the current tile; past its end it names a slab of the next tile.
-  auto touch_ahead = [&](const Desc& cur_d, const Desc& next_d, bool have_next, int s) {
-    if (s < kt_n) touch_slab(cur_d, s);
-    else if (have_next) touch_slab(next_d, s - kt_n);
   };
 
   // Epilogue staging: a private region per wave inside slab buffer NSTAGE-1 (free between tiles),
   // 32 rows x (BN/WN) columns of 16-bit outputs, rows padded by 16 bytes.
   char* const stage_c = smem + (C::NSTAGE - 1) * C::STAGE_BYTES + wave * C::EPI_WAVE_BYTES;
 
-  int64_t tile_id = sched_first_tile(p.tile_order);
+  int64_t tile_id = sched_first_tile();
   Tile t;
-  Desc dsc = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+  TileIo io;
   if (tile_id < num_tiles) {
     t = sched_tile<C::BM, C::BN>(p, sched, tile_id);
-    dsc = make_desc(t);
+    io = make_io(t);
 #pragma unroll
-    for (int s = 0; s < C::NSTAGE - 1; ++s) {
-      issue_slab(dsc, s, s);
-      touch_slab(dsc, s + C::PFD);
-    }
+    for (int s = 0; s < C::NSTAGE - 1; ++s) issue_slab(io, s, s);
   }
   while (tile_id < num_tiles) {
-    // look one tile ahead: its descriptors are needed for warm-up reads near the end of this tile
-    const int64_t next_id = tile_id + gridDim.x;
-    const bool have_next = next_id < num_tiles;
-    Tile nt = t;
-    Desc ndsc = dsc;
-    if (have_next) {
-      nt = sched_tile<C::BM, C::BN>(p, sched, next_id);
-      ndsc = make_desc(nt);
-    }
-
     f32x16_t acc[C::TM][C::TN];
 #pragma unroll
     for (int i = 0; i < C::TM; ++i)
@@ -223,56 +255,66 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_nt_kernel(const GemmPara
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
+    const int kt_n = io.kt_n;
     for (int kt = 0; kt < kt_n; ++kt) {
-      if (copier) wait_vmcnt<C::LPW * (C::NSTAGE - 2)>();  // this wave's share of slab kt has landed
-      __syncthreads();  // everyone's share of slab kt has landed; everyone is done with slab kt-1
-      issue_slab(dsc, kt + C::NSTAGE - 1, (kt + C::NSTAGE - 1) % C::NSTAGE);
-      touch_ahead(dsc, ndsc, have_next, kt + C::NSTAGE - 1 + C::PFD);
-      const char* sa = smem + (kt % C::NSTAGE) * C::STAGE_BYTES + wm0 * C::RB;
-      const char* sb = smem + (kt % C::NSTAGE) * C::STAGE_BYTES + C::A_BYTES + wn0 * C::RB;
+      wait_vmcnt<C::LPW * (C::NSTAGE - 2)>();  // this wave's share of slab kt has landed
+      __syncthreads();                          // everyone's share has; everyone is done with slab kt-1
+      issue_slab(io, kt + C::NSTAGE - 1, (kt + C::NSTAGE - 1) % C::NSTAGE);
+      const char* sa = smem + (kt % C::NSTAGE) * C::STAGE_BYTES;
+      const char* sb = sa + C::A_BYTES;
 #pragma unroll
-      for (int ks = 0; ks < C::BK / 16; ++ks) {
+      for (int ks = 0; ks < BK / 16; ++ks) {
         i32x4_t fa[C::TM], fb[C::TN];
 #pragma unroll
         for (int i = 0; i < C::TM; ++i) {
-          if (DBG & 2) { fa[i][0] = kt + i; fa[i][1] = ks; fa[i][2] = lane; fa[i][3] = i; }
-          else fa[i] = *(const i32x4_t*)(sa + rd_off[ks] + i * 32 * C::RB);
+          if (A_KMAJOR) {
+            fa[i] = *(const i32x4_t*)(sa + a_rd[ks] + i * 32 * 128);
+          } else {
+            const char* q = sa + a_rd[i] + ks * 16 * (C::BM * 2);
+            const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)q);
+            const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)(q + 4 * (C::BM * 2)));
+            fa[i] = __builtin_bit_cast(i32x4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+          }
         }
 #pragma unroll
         for (int j = 0; j < C::TN; ++j) {
-          if (DBG & 2) { fb[j][0] = kt; fb[j][1] = ks + j; fb[j][2] = lane; fb[j][3] = j; }
-          else fb[j] = *(const i32x4_t*)(sb + rd_off[ks] + j * 32 * C::RB);
+          if (B_KMAJOR) {
+            fb[j] = *(const i32x4_t*)(sb + b_rd[ks] + j * 32 * 128);
+          } else {
+            const char* q = sb + b_rd[j] + ks * 16 * (C::BN * 2);
+            const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)q);
+            const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)(q + 4 * (C::BN * 2)));
+            fb[j] = __builtin_bit_cast(i32x4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+          }
         }
 #pragma unroll
         for (int i = 0; i < C::TM; ++i)
 #pragma unroll
-          for (int j = 0; j < C::TN; ++j) {
-            if (DBG & 4) { acc[i][j][0] += __builtin_bit_cast(float, fa[i][0] ^ fb[j][1]); acc[i][j][5] += __builtin_bit_cast(float, fa[i][3] ^ fb[j][2]); }
-            else acc[i][j] = Mma16<DT>::run(fb[j], fa[i], acc[i][j]);
-          }
+          for (int j = 0; j < C::TN; ++j) acc[i][j] = Mma16<DT>::run(fb[j], fa[i], acc[i][j]);
       }
     }
-    if (copier) wait_vmcnt<0>();
+    wait_vmcnt<0>();
     __syncthreads();  // every fragment read of this tile is done: all slab buffers are free
 
-    // Start the next tile's first slabs before draining this tile's results (they were warmed by the
-    // touches of this tile's last iterations).
+    // Request the next tile's first slabs before draining this tile's results.
     const Tile cur = t;
-    if (have_next) {
-      t = nt;
-      dsc = ndsc;
+    const int64_t next_id = tile_id + gridDim.x;
+    if (next_id < num_tiles) {
+      t = sched_tile<C::BM, C::BN>(p, sched, next_id);
+      io = make_io(t);
 #pragma unroll
-      for (int s = 0; s < C::NSTAGE - 1; ++s) issue_slab(dsc, s, s);
+      for (int s = 0; s < C::NSTAGE - 1; ++s) issue_slab(io, s, s);
     }
     tile_id = next_id;
 
     // Epilogue.  A lane owns row l32 and columns 32 j + 8 q + 4 lh + (0..3) of each 32-row block i:
-    // transpose through the wave's LDS staging so that global stores are 16 bytes per lane and
-    // whole 128-byte (or longer) row segments per instruction.
-    constexpr int WCOLS = C::BN / C::WN;          // columns owned by this wave
-    constexpr int CPRW = WCOLS / 8;               // 16-byte chunks per staged row
-    constexpr int RPIW = 64 / CPRW;               // rows covered by one wave-wide read
-    char* const c_tile = (char*)p.C + ((cur.row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2;
+    // transpose through the wave's LDS staging so that global stores are 16 bytes per lane and whole
+    // 128-byte (or longer) row segments per instruction.
+    constexpr int WCOLS = C::BN / C::WN;  // columns owned by this wave
+    constexpr int CPRW = WCOLS / 8;       // 16-byte chunks per staged row
+    constexpr int RPIW = 64 / CPRW;       // rows covered by one wave-wide read
+    const int64_t c_row0 = (LAYOUT == LAYOUT_TN) ? ((int64_t)cur.g * p.m_total + cur.row0) : cur.row0;
+    char* const c_tile = (char*)p.C + ((c_row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2;
     const int st_row = lane / CPRW, st_chunk = lane % CPRW;
     const bool col_ok = cur.n0 + wn0 + st_chunk * 8 < p.N;
 #pragma unroll
@@ -294,14 +336,12 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_nt_kernel(const GemmPara
   }
 }
 
-int g_tile_order = 0;
-
-template <class C, int DT, int DBG = 0>
+template <class C, int DT, int LAYOUT>
 int launch_cfg(const GemmParams& p, hipStream_t s) {
   static bool attr_set[64] = {false};
   int dev = 0;
   (void)hipGetDevice(&dev);
-  auto kern = gemm_fast_nt_kernel<C, DT, DBG>;
+  auto kern = gemm_fast_kernel<C, DT, LAYOUT>;
   if (dev >= 0 && dev < 64 && !attr_set[dev]) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM_BYTES) != hipSuccess)
       return check_launch("hipFuncSetAttribute(gemm_fast)");
@@ -309,61 +349,56 @@ int launch_cfg(const GemmParams& p, hipStream_t s) {
   }
   int grid = num_cus();
   if (p.grid_limit > 0 && p.grid_limit < grid) grid = p.grid_limit;
-  GemmParams q = p;
-  q.tile_order = g_tile_order;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::THREADS), C::SMEM_BYTES, s, q);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::THREADS), C::SMEM_BYTES, s, p);
   return check_launch("gemm_fast");
 }
 
 int g_variant = 0;
 
-template <int DT>
+template <int DT, int LAYOUT>
 int launch_variant(const GemmParams& p, hipStream_t s) {
   switch (g_variant) {
     default:
-    case 0: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 4>, DT>(p, s);
-    case 1: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 2>, DT>(p, s);
-    case 2: return launch_cfg<FastCfg<256, 128, 64, 3, 4, 2>, DT>(p, s);
-    case 3: return launch_cfg<FastCfg<256, 128, 64, 3, 2, 2>, DT>(p, s);
-    case 4: return launch_cfg<FastCfg<256, 128, 64, 3, 2, 4>, DT>(p, s);
-    case 5: return launch_cfg<FastCfg<128, 256, 64, 3, 2, 2>, DT>(p, s);
-    case 6: return launch_cfg<FastCfg<256, 128, 64, 2, 2, 4>, DT>(p, s);
-    case 7: return launch_cfg<FastCfg<128, 128, 64, 4, 2, 2>, DT>(p, s);
-    case 8: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 4, 0>, DT>(p, s);
-    case 9: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 4, 3>, DT>(p, s);
-    case 16: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 4, 1>, DT>(p, s);
-    case 17: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 4, 4>, DT>(p, s);
-    case 10: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 4>, DT, 1>(p, s);
-    case 11: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 4>, DT, 2>(p, s);
-    case 12: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 4>, DT, 4>(p, s);
-    case 13: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 4>, DT, 3>(p, s);
-    case 14: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 4>, DT, 6>(p, s);
-    case 15: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 4>, DT, 5>(p, s);
-    case 20: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 2>, DT, 1>(p, s);
-    case 21: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 2>, DT, 2>(p, s);
-    case 23: return launch_cfg<FastCfg<256, 256, 64, 2, 2, 2>, DT, 3>(p, s);
+    case 0: return launch_cfg<FastCfg<256, 256, 2, 2, 4>, DT, LAYOUT>(p, s);
+    case 1: return launch_cfg<FastCfg<256, 128, 3, 4, 2>, DT, LAYOUT>(p, s);
+    case 2: return launch_cfg<FastCfg<256, 128, 3, 2, 4>, DT, LAYOUT>(p, s);
+    case 3: return launch_cfg<FastCfg<128, 256, 3, 2, 4>, DT, LAYOUT>(p, s);
+    case 4: return launch_cfg<FastCfg<128, 128, 4, 2, 2>, DT, LAYOUT>(p, s);
   }
+}
+
+template <int DT>
+int launch_layout(const GemmParams& p, int layout, hipStream_t s) {
+  if (layout == LAYOUT_NT) return launch_variant<DT, LAYOUT_NT>(p, s);
+  if (layout == LAYOUT_NN) return launch_variant<DT, LAYOUT_NN>(p, s);
+  return launch_variant<DT, LAYOUT_TN>(p, s);
 }
 
 }  // namespace
 
 void set_fast_variant(int v) { g_variant = v; }
-void set_tile_order(int v) { g_tile_order = v; }
+void set_tile_order(int) {}
 
 bool fast_supported(const GemmParams& p, int dt, int layout) {
-  if (layout != 0) return false;
   if (dt != DT_BF16 && dt != DT_F16) return false;
-  if (p.mode != MODE_MG && p.mode != MODE_MG_PAD && p.mode != MODE_MASKED) return false;
   if (p.G > kFastMaxGroups) return false;
-  if (p.K < 64 || (p.K % 64) != 0) return false;
-  if ((int64_t)p.K * 2 * 256 >= (1ll << 30)) return false;  // slab offsets stay far below the out-of-range marker
-  return true;
+  if ((p.N & 7) != 0) return false;
+  if (layout == LAYOUT_TN) {
+    if (p.mode != MODE_KG) return false;
+    if ((p.m_total & 7) != 0) return false;
+    return p.m_total * 2 * 64 < (1ll << 30) && (int64_t)p.N * 2 * 64 < (1ll << 30);
+  }
+  if (p.mode != MODE_MG && p.mode != MODE_MG_PAD && p.mode != MODE_MASKED) return false;
+  if (p.K < BK || (p.K % BK) != 0) return false;
+  // per-lane source offsets stay far below the out-of-range marker
+  if ((int64_t)p.K * 2 * 256 >= (1ll << 30)) return false;
+  if (layout == LAYOUT_NN && (int64_t)p.N * 2 * 64 >= (1ll << 30)) return false;
+  return layout == LAYOUT_NT || layout == LAYOUT_NN;
 }
 
 int launch_fast_16bit(const GemmParams& p, int dt, int layout, hipStream_t s) {
-  (void)layout;
-  if (dt == DT_BF16) return launch_variant<DT_BF16>(p, s);
-  return launch_variant<DT_F16>(p, s);
+  if (dt == DT_BF16) return launch_layout<DT_BF16>(p, layout, s);
+  return launch_layout<DT_F16>(p, layout, s);
 }
 
 }  // namespace tgg
