@@ -101,7 +101,7 @@ def build_workload(name: str, dev, seed: int = 2026):
         from triton_grouped_gemm_amd.gemm.deep_gemm_ops import m_grouped_fp8_nt_contiguous
         from triton_grouped_gemm_amd.quant.fp8_cast import per_block_cast_to_fp8, per_token_cast_to_fp8
         a = wl.randn_bf16((M_TOTAL, K), 1.0, seed + 1, dev)
-        aq = per_token_cast_to_fp8(a)
+        aq = per_token_cast_to_fp8(a, scales_mn_major=True)
         del a
         w = wl.randn_bf16((G, N, K), 1.0, seed + 2, dev)
         wq = per_block_cast_to_fp8(w)

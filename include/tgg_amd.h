@@ -67,12 +67,13 @@ int tgg_k_grouped_gemm_fp8_channel(const void* x, const float* xs, const void* y
                                    int num_cu, void* stream);
 
 /* out[r,n] = sum_kb (sum_{k in kb} Aq[r,k] Bq[g,n,k]) * sa[r,kb] * sb[g,n/128,kb]; e4m3fn codes, A physically
- * padded per group to `align` rows, sa [M,ceil(K/128)], sb [G,ceil(N/128),ceil(K/128)], bf16 output.
- * Replaces deep_gemm.m_grouped_fp8_gemm_nt_contiguous as called from m_grouped_fp8_nt_contiguous
+ * padded per group to `align` rows, sb [G,ceil(N/128),ceil(K/128)], bf16 output.  sa holds M x ceil(K/128)
+ * floats, row-major [M,KB] (sa_mn_major=0) or KB-major [KB,M] (sa_mn_major=1, the layout the tuned kernel
+ * streams).  Replaces deep_gemm.m_grouped_fp8_gemm_nt_contiguous as called from m_grouped_fp8_nt_contiguous
  * (gemm/deep_gemm_ops.py:60-100). */
 int tgg_m_grouped_gemm_fp8_block(const void* Aq, const float* sa, const void* Bq, const float* sb, void* C,
                                  const void* sizes, int sizes_i64, int G, int64_t M, int N, int K, int align,
-                                 int num_cu, void* stream);
+                                 int sa_mn_major, int num_cu, void* stream);
 
 /* bf16 x [M,N] -> codes [N,M_expand] (transposed, each group padded to 128 columns, zero tail) and
  * scales [N/128, M_expand/128].  Replaces trans_per_block_quant_expand_128x
@@ -81,9 +82,11 @@ int tgg_trans_per_block_quant_expand_128x(const void* x, void* codes, float* sca
                                           int sizes_i64, int G, int64_t M, int N, int64_t M_expand, int fmt,
                                           void* stream);
 
-/* bf16 x [M,K] -> codes [M,K], scales [M,K/128]; 1x128 recipe.  Replaces per_token_cast_to_fp8
+/* bf16 x [M,K] -> codes [M,K], scales [M,K/128] (scales_mn_major=0) or stored transposed [K/128,M]
+ * (scales_mn_major=1); 1x128 recipe.  Replaces per_token_cast_to_fp8
  * (gemm/FP8/m_grouped_gemm_channel_expert.py:217-222). */
-int tgg_per_token_cast_to_fp8(const void* x, void* codes, float* scales, int64_t M, int K, int fmt, void* stream);
+int tgg_per_token_cast_to_fp8(const void* x, void* codes, float* scales, int64_t M, int K, int fmt,
+                              int scales_mn_major, void* stream);
 
 /* bf16 x [batch,R,C] -> codes (same shape), scales [batch,ceil(R/128),ceil(C/128)]; 128x128 recipe.
  * Replaces per_block_cast_to_fp8 (gemm/FP8/m_grouped_gemm_channel_expert.py:237-245). */
@@ -95,7 +98,7 @@ int tgg_per_block_cast_to_fp8(const void* x, void* codes, float* scales, int bat
 int tgg_cvt_f32_to_fp8(const float* in, void* out, int64_t n, int fmt, void* stream);
 
 /* Library controls: "force_generic" (0/1) routes every GEMM through the shape-agnostic kernel;
- * "variant" (int) selects a tile configuration of the tuned kernels (0 = default). */
+ * "variant" (int) selects a tile configuration of the tuned 16-bit kernels (0 = default). */
 int tgg_set_option(const char* key, int value);
 const char* tgg_last_error(void);
 int tgg_version(void);

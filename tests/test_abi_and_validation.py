@@ -45,7 +45,7 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert lib.tgg_m_grouped_gemm(p + 4, p, p, p, 0, 4, 128, 128, 128, 1, 0, -1, None) == 1
     assert "aligned" in _native.last_error()
     assert lib.tgg_trans_per_block_quant_expand_128x(p, p, p, p, 0, 2, 256, 100, 512, 2, None) == 1
-    assert lib.tgg_per_token_cast_to_fp8(p, p, p, 4, 100, 2, None) == 1
+    assert lib.tgg_per_token_cast_to_fp8(p, p, p, 4, 100, 2, 0, None) == 1
     assert lib.tgg_set_option(b"nope", 1) == 1
     assert lib.tgg_set_option(b"force_generic", 0) == 0
 

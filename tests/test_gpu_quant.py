@@ -100,6 +100,9 @@ def test_per_token_cast_bit_exact(dev, dtype):
     rc, rs = quant_ref.per_token_cast_to_fp8(to_np_f32(x), FMT[dtype])
     assert np.array_equal(scales.cpu().numpy().view(np.uint32), rs.view(np.uint32))
     assert np.array_equal(codes_np(codes), rc)
+    codes2, scales2 = per_token_cast_to_fp8(x.to(dev), dtype, scales_mn_major=True)
+    assert scales2.shape == scales.shape and scales2.stride() == (1, 300)
+    assert torch.equal(scales2, scales) and torch.equal(codes2.view(torch.uint8), codes.view(torch.uint8))
 
 
 @pytest.mark.parametrize("shape", [(256, 384), (130, 200), (3, 136, 264), (2, 128, 128)])

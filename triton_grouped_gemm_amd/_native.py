@@ -26,9 +26,9 @@ SIGNATURES = {
     "tgg_k_grouped_gemm": [_P, _P, _P, _P, _P, _I, _I, _I, _L, _I, _I, _P],
     "tgg_m_grouped_gemm_fp8_channel": [_P, _P, _P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _I, _I, _P],
     "tgg_k_grouped_gemm_fp8_channel": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _L, _I, _I, _I, _P],
-    "tgg_m_grouped_gemm_fp8_block": [_P, _P, _P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _P],
+    "tgg_m_grouped_gemm_fp8_block": [_P, _P, _P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _I, _P],
     "tgg_trans_per_block_quant_expand_128x": [_P, _P, _P, _P, _I, _I, _L, _I, _L, _I, _P],
-    "tgg_per_token_cast_to_fp8": [_P, _P, _P, _L, _I, _I, _P],
+    "tgg_per_token_cast_to_fp8": [_P, _P, _P, _L, _I, _I, _I, _P],
     "tgg_per_block_cast_to_fp8": [_P, _P, _P, _I, _I, _I, _I, _P],
     "tgg_cvt_f32_to_fp8": [_P, _P, _L, _I, _P],
     "tgg_set_option": [c_char_p, _I],

@@ -40,13 +40,12 @@ int num_cus() {
 }
 
 int launch_trans_quant128(const void*, void*, float*, const GemmParams&, int64_t, int, hipStream_t);
-int launch_token_cast128(const void*, void*, float*, int64_t, int, hipStream_t);
+int launch_token_cast128(const void*, void*, float*, int64_t, int, int, int, hipStream_t);
 int launch_block_cast128(const void*, void*, float*, int, int, int, int, hipStream_t);
 int launch_cvt_fp8(const float*, void*, int64_t, int, hipStream_t);
 bool fast_supported(const GemmParams& p, int dt, int layout);
 int launch_fast_16bit(const GemmParams& p, int dt, int layout, hipStream_t s);
 void set_fast_variant(int v);
-void set_tile_order(int v);
 
 static bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 
@@ -158,6 +157,7 @@ int tgg_m_grouped_gemm_fp8_channel(const void* Aq, const float* a_scale, const v
   p.mode = MODE_MG; p.m_total = M; p.N = N; p.K = K;
   p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K; p.b_sn = K; p.b_sk = 1;
   p.grid_limit = num_cu;
+  if (!g_force_generic && fast_fp8_supported(p, false)) return launch_fast_fp8_channel(p, fmt_a, fmt_b, out_dtype, (hipStream_t)stream);
   return launch_generic_fp8_channel(p, fmt_a, fmt_b, out_dtype, (hipStream_t)stream);
 }
 
@@ -175,12 +175,13 @@ int tgg_k_grouped_gemm_fp8_channel(const void* x, const float* xs, const void* y
   p.mode = MODE_KG_COUNT; p.m_total = M; p.k_total = Ktot; p.N = N; p.K = 0;
   p.a_sm = Ktot; p.a_sk = 1; p.b_sg = 0; p.b_sn = Ktot; p.b_sk = 1; p.c_sg = (int64_t)M * N;
   p.grid_limit = num_cu;
+  if (!g_force_generic && fast_fp8_supported(p, false)) return launch_fast_fp8_channel(p, fmt_a, fmt_b, TGG_BF16, (hipStream_t)stream);
   return launch_generic_fp8_channel(p, fmt_a, fmt_b, TGG_BF16, (hipStream_t)stream);
 }
 
 int tgg_m_grouped_gemm_fp8_block(const void* Aq, const float* sa, const void* Bq, const float* sb, void* C,
                                  const void* sizes, int sizes_i64, int G, int64_t M, int N, int K, int align,
-                                 int num_cu, void* stream) {
+                                 int sa_mn_major, int num_cu, void* stream) {
   if (int e = check_common(Aq, Bq, C, sizes, G, N)) return e;
   if (!sa || !sb) return set_error("null scale pointer");
   if (M < 0 || K < 0) return set_error("negative M or K");
@@ -190,9 +191,13 @@ int tgg_m_grouped_gemm_fp8_block(const void* Aq, const float* sa, const void* Bq
   GemmParams p = zero_params();
   p.A = Aq; p.B = Bq; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
   p.sa = sa; p.sb = sb;
+  const int kblocks = (K + 127) / 128;
+  if (sa_mn_major) { p.sa_rs = 1; p.sa_ks = M; } else { p.sa_rs = kblocks; p.sa_ks = 1; }
   p.mode = MODE_MG_PAD; p.align = align; p.m_total = M; p.N = N; p.K = K;
   p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K; p.b_sn = K; p.b_sk = 1;
   p.grid_limit = num_cu;
+  if (!g_force_generic && sa_mn_major && kblocks <= 64 && fast_fp8_supported(p, true))
+    return launch_fast_fp8_block(p, (hipStream_t)stream);
   return launch_generic_fp8_block(p, (hipStream_t)stream);
 }
 
@@ -211,11 +216,12 @@ int tgg_trans_per_block_quant_expand_128x(const void* x, void* codes, float* sca
   return launch_trans_quant128(x, codes, scales, p, M_expand, fmt, (hipStream_t)stream);
 }
 
-int tgg_per_token_cast_to_fp8(const void* x, void* codes, float* scales, int64_t M, int K, int fmt, void* stream) {
+int tgg_per_token_cast_to_fp8(const void* x, void* codes, float* scales, int64_t M, int K, int fmt,
+                              int scales_mn_major, void* stream) {
   if (!x || !codes || !scales) return set_error("null pointer");
   if (M < 0 || K < 0 || (K & 127)) return set_error("K must be a multiple of 128, got %d", K);
   if (!aligned16(x) || !aligned16(codes)) return set_error("operand pointers must be 16-byte aligned");
-  return launch_token_cast128(x, codes, scales, M * (K / 128), fmt, (hipStream_t)stream);
+  return launch_token_cast128(x, codes, scales, M, K / 128, scales_mn_major, fmt, (hipStream_t)stream);
 }
 
 int tgg_per_block_cast_to_fp8(const void* x, void* codes, float* scales, int batch, int R, int C, int fmt,
@@ -234,7 +240,6 @@ int tgg_cvt_f32_to_fp8(const float* in, void* out, int64_t n, int fmt, void* str
 int tgg_set_option(const char* key, int value) {
   if (key && strcmp(key, "force_generic") == 0) { g_force_generic = value != 0; return 0; }
   if (key && strcmp(key, "variant") == 0) { set_fast_variant(value); return 0; }
-  if (key && strcmp(key, "tile_order") == 0) { set_tile_order(value); return 0; }
   return set_error("unknown option '%s'", key ? key : "(null)");
 }
 

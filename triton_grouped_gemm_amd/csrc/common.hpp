@@ -67,7 +67,7 @@ struct GemmParams {
   const int32_t* k_end;   // MODE_KG only
   const float* scale_m;   // per-row scale (channel modes) or nullptr
   const float* scale_n;   // per-(group, column) scale, indexed g*N + n, or nullptr
-  const float* sa;        // block-scaled: [rows, ceil(K/128)] activation scales
+  const float* sa;        // block-scaled activation scales: element (row, kb) at row * sa_rs + kb * sa_ks
   const float* sb;        // block-scaled: [G, ceil(N/128), ceil(K/128)] weight scales
   int64_t m_total;        // rows of A/C that may be touched (M-grouped), Mdim for K-grouped
   int64_t m_stride;       // MODE_MASKED: rows between consecutive groups
@@ -76,6 +76,7 @@ struct GemmParams {
   int64_t b_sg, b_sn, b_sk;
   int64_t c_sg;           // K-grouped: elements between consecutive groups' outputs
   int64_t scale_m_sg;     // K-grouped channel mode: scale_m stride between groups
+  int64_t sa_rs, sa_ks;   // strides (in floats) of the block-scaled activation scales
   int sizes_i64;
   int G;
   int mode;
@@ -83,7 +84,6 @@ struct GemmParams {
   int N;
   int K;                  // reduction length (M-grouped); unused for K-grouped
   int grid_limit;         // >0 caps the persistent grid
-  int tile_order;         // 0: XCD-contiguous tile runs, 1: plain round robin
 };
 
 }  // namespace tgg

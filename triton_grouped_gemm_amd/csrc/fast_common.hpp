@@ -1,0 +1,73 @@
+// Building blocks shared by the tuned gfx950 GEMM kernels: direct-to-LDS slab copies, their buffer
+// descriptors, the vmcnt bookkeeping and the swizzled slab geometry.
+#pragma once
+#include "common.hpp"
+#include "sched.hpp"
+
+namespace tgg {
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __attribute__((address_space(3))) i16x4_t* lds_i16x4_ptr_t;
+
+// s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]).
+template <int N> TGG_DEV void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt range");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+// One wave-wide 16-byte-per-lane copy global -> LDS.  The LDS destination is m0 + lane * 16, the
+// global source is the descriptor base + voff (bounds-checked: out-of-range lanes write zeros).
+// Written as inline assembly on purpose: the compiler does not model the copy, so it cannot
+// serialise the software pipeline with conservative waits; completion is tracked by hand with
+// wait_vmcnt<>() and the workgroup barrier.
+TGG_DEV void copy_b128_to_lds(i32x4_t rsrc, uint32_t lds_addr, int voff) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
+}
+
+// A run of slabs of one operand: slab kt starts at base + kt * step and may touch `bytes - kt * step`
+// bytes from there (everything beyond reads as zero).  All fields are wave-uniform.
+struct Stream {
+  uint64_t base;
+  int64_t bytes;
+  int64_t step;
+};
+
+TGG_DEV i32x4_t stream_rsrc(const Stream& s, int kt) {
+  const uint64_t a = s.base + (uint64_t)(kt * s.step);
+  int64_t left = s.bytes - kt * s.step;
+  left = left < 0 ? 0 : (left > 0x7fffffff ? 0x7fffffff : left);
+  i32x4_t r;  // readfirstlane pins the descriptor to scalar registers
+  r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
+  r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32) & 0xffff);  // stride 0, no swizzle
+  r[2] = __builtin_amdgcn_readfirstlane((int)left);
+  r[3] = 0x00020000;  // raw buffer, 32-bit data format
+  return r;
+}
+
+constexpr int kFastMaxGroups = 256;
+constexpr int kSlabRowBytes = 128;  // a slab holds 128 bytes of every K-contiguous row (64 bf16 / 128 fp8 values)
+
+// Geometry of one operand's slab in LDS and of the copies that fill it.
+//   KMAJOR: ROWS rows of 128 bytes (64 K values each).  A copy instruction covers 8 rows; the
+//           16-byte chunk c of row r sits at slot c ^ ((r / 2) % 8).
+//   !KMAJOR: 64 token rows of ROWS*2 bytes.  A copy instruction covers 1024 / (ROWS*2) token rows;
+//           chunk c of token row k sits at slot c ^ ((k % 4) * 4).
+template <int ROWS, bool KMAJOR> struct Operand {
+  static constexpr int SLAB_BYTES = ROWS * kSlabRowBytes;
+  static constexpr int NI = SLAB_BYTES / 1024;                 // copy instructions per slab
+  static constexpr int ROW_BYTES = KMAJOR ? kSlabRowBytes : ROWS * 2;  // bytes of one LDS row (token rows: 16-bit)
+  static constexpr int CPR = ROW_BYTES / 16;                   // 16-byte chunks per LDS row
+  static constexpr int RPI = 1024 / ROW_BYTES;                 // LDS rows per copy instruction
+  static constexpr int NPAT = KMAJOR ? 2 : (RPI >= 4 ? 1 : 4 / RPI);  // swizzle patterns over instructions
+
+  // byte offset (from the slab's first byte in global memory) fetched by `lane` of a copy
+  // instruction with swizzle pattern `pat`; ld = bytes between consecutive global rows.
+  static TGG_DEV int lane_voff(int lane, int pat, int ld) {
+    const int r_local = lane / CPR, slot = lane % CPR;
+    const int r = pat * RPI + r_local;  // row index modulo the swizzle period
+    const int sw = KMAJOR ? (r / 2) % 8 : (r % 4) * 4;
+    return r_local * ld + ((slot ^ sw) << 4);
+  }
+};
+
+}  // namespace tgg

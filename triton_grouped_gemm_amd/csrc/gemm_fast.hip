@@ -21,18 +21,15 @@
 //     srcA and the A operand as srcB, so a lane ends up with 4 consecutive output columns of one
 //     row; results are transposed through a per-wave LDS staging area and leave as 16-byte stores
 //     covering whole 128-byte row segments.
-#include "common.hpp"
-#include "sched.hpp"
+#include "fast_common.hpp"
 #include "launch.hpp"
 
 namespace tgg {
 
 namespace {
 
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-typedef __attribute__((address_space(3))) i16x4_t* lds_i16x4_ptr_t;
-
 enum : int { LAYOUT_NT = 0, LAYOUT_NN = 1, LAYOUT_TN = 2 };
+constexpr int BK = 64;  // K depth of a slab for 16-bit operands
 
 template <int DT> struct Mma16;
 template <> struct Mma16<DT_BF16> {
@@ -43,67 +40,6 @@ template <> struct Mma16<DT_BF16> {
 template <> struct Mma16<DT_F16> {
   static TGG_DEV f32x16_t run(i32x4_t w, i32x4_t x, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, w), __builtin_bit_cast(f16x8_t, x), c, 0, 0, 0);
-  }
-};
-
-// s_waitcnt vmcnt(n) only (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]).
-template <int N> TGG_DEV void wait_vmcnt() {
-  static_assert(N >= 0 && N < 64, "vmcnt range");
-  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
-
-// One wave-wide 16-byte-per-lane copy global -> LDS.  The LDS destination is m0 + lane * 16, the
-// global source is the descriptor base + voff (bounds-checked: out-of-range lanes write zeros).
-// Written as inline assembly on purpose: the compiler does not model the copy, so it cannot
-// serialise the software pipeline with conservative waits; completion is tracked by hand with
-// wait_vmcnt<>() and the workgroup barrier.
-TGG_DEV void copy_b128_to_lds(i32x4_t rsrc, uint32_t lds_addr, int voff) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
-}
-
-// A run of slabs of one operand: slab kt starts at base + kt * step and may touch `bytes - kt * step`
-// bytes from there (everything beyond reads as zero).  All fields are wave-uniform.
-struct Stream {
-  uint64_t base;
-  int64_t bytes;
-  int64_t step;
-};
-
-TGG_DEV i32x4_t stream_rsrc(const Stream& s, int kt) {
-  const uint64_t a = s.base + (uint64_t)(kt * s.step);
-  int64_t left = s.bytes - kt * s.step;
-  left = left < 0 ? 0 : (left > 0x7fffffff ? 0x7fffffff : left);
-  i32x4_t r;  // readfirstlane pins the descriptor to scalar registers
-  r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
-  r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32) & 0xffff);  // stride 0, no swizzle
-  r[2] = __builtin_amdgcn_readfirstlane((int)left);
-  r[3] = 0x00020000;  // raw buffer, 32-bit data format
-  return r;
-}
-
-constexpr int kFastMaxGroups = 256;
-constexpr int BK = 64;  // K depth of a slab: 128 bytes of a K-contiguous row
-
-// Geometry of one operand's slab in LDS and of the copies that fill it.
-//   KMAJOR: ROWS rows of 128 bytes (64 K values each).  A copy instruction covers 8 rows; the
-//           16-byte chunk c of row r sits at slot c ^ ((r / 2) % 8).
-//   !KMAJOR: 64 token rows of ROWS*2 bytes.  A copy instruction covers 1024 / (ROWS*2) token rows;
-//           chunk c of token row k sits at slot c ^ ((k % 4) * 4).
-template <int ROWS, bool KMAJOR> struct Operand {
-  static constexpr int SLAB_BYTES = ROWS * BK * 2;
-  static constexpr int NI = SLAB_BYTES / 1024;                 // copy instructions per slab
-  static constexpr int ROW_BYTES = KMAJOR ? BK * 2 : ROWS * 2; // bytes of one LDS row
-  static constexpr int CPR = ROW_BYTES / 16;                   // 16-byte chunks per LDS row
-  static constexpr int RPI = 1024 / ROW_BYTES;                 // LDS rows per copy instruction
-  static constexpr int NPAT = KMAJOR ? 2 : (RPI >= 4 ? 1 : 4 / RPI);  // swizzle patterns over instructions
-
-  // byte offset (from the slab's first byte in global memory) fetched by `lane` of a copy
-  // instruction with swizzle pattern `pat`; ld = bytes between consecutive global rows.
-  static TGG_DEV int lane_voff(int lane, int pat, int ld) {
-    const int r_local = lane / CPR, slot = lane % CPR;
-    const int r = pat * RPI + r_local;  // row index modulo the swizzle period
-    const int sw = KMAJOR ? (r / 2) % 8 : (r % 4) * 4;
-    return r_local * ld + ((slot ^ sw) << 4);
   }
 };
 
@@ -377,7 +313,6 @@ int launch_layout(const GemmParams& p, int layout, hipStream_t s) {
 }  // namespace
 
 void set_fast_variant(int v) { g_variant = v; }
-void set_tile_order(int) {}
 
 bool fast_supported(const GemmParams& p, int dt, int layout) {
   if (dt != DT_BF16 && dt != DT_F16) return false;

@@ -216,7 +216,7 @@ __global__ __launch_bounds__(GTHREADS) void gemm_generic_kernel(const GemmParams
 #pragma unroll
           for (int i = 0; i < 2; ++i) {
             const int m = wm + i * 32 + l32;
-            const float s = (m < t.rows) ? p.sa[(t.row0 + m) * kblocks + kb] * sbv : 0.f;
+            const float s = (m < t.rows) ? p.sa[(t.row0 + m) * p.sa_rs + kb * p.sa_ks] * sbv : 0.f;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll

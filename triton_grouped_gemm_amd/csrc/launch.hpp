@@ -15,5 +15,8 @@ struct GemmParams;
 int launch_generic_16bit(const GemmParams& p, int dt, int layout, hipStream_t s);
 int launch_generic_fp8_channel(const GemmParams& p, int ta, int tb, int out_dt, hipStream_t s);
 int launch_generic_fp8_block(const GemmParams& p, hipStream_t s);
+bool fast_fp8_supported(const GemmParams& p, bool block_scaled);
+int launch_fast_fp8_channel(const GemmParams& p, int ta, int tb, int out_dt, hipStream_t s);
+int launch_fast_fp8_block(const GemmParams& p, hipStream_t s);
 
 }  // namespace tgg

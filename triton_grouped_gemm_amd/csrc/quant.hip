@@ -138,8 +138,9 @@ __global__ __launch_bounds__(256) void trans_quant128_kernel(const uint16_t* __r
 // 16 lanes per 1x128 group; each lane 8 elements.
 template <int FMT>
 __global__ __launch_bounds__(256) void token_cast128_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ codes,
-                                                           float* __restrict__ scales, int64_t groups) {
+                                                           float* __restrict__ scales, int64_t rows, int kblocks, int mn_major) {
   constexpr float fmax_ = FmtMax<FMT>::v;
+  const int64_t groups = rows * kblocks;
   const int sub = threadIdx.x & 15;
   for (int64_t g = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4); g < groups; g += (int64_t)gridDim.x * 16) {
     const i32x4_t v = *(const i32x4_t*)(x + g * 128 + sub * 8);
@@ -159,7 +160,7 @@ __global__ __launch_bounds__(256) void token_cast128_kernel(const uint16_t* __re
     pk.x = cvt4<FMT>(f[0], f[1], f[2], f[3]);
     pk.y = cvt4<FMT>(f[4], f[5], f[6], f[7]);
     *(uint2*)(codes + g * 128 + sub * 8) = pk;
-    if (sub == 0) scales[g] = amax / fmax_;
+    if (sub == 0) scales[mn_major ? (g % kblocks) * rows + g / kblocks : g] = amax / fmax_;
   }
 }
 
@@ -258,17 +259,19 @@ int launch_trans_quant128(const void* x, void* codes, float* scales, const GemmP
   return check_launch("trans_quant128");
 }
 
-int launch_token_cast128(const void* x, void* codes, float* scales, int64_t groups, int fmt, hipStream_t s) {
+int launch_token_cast128(const void* x, void* codes, float* scales, int64_t rows, int kblocks, int mn_major, int fmt,
+                         hipStream_t s) {
+  const int64_t groups = rows * kblocks;
   if (groups == 0) return 0;
   int64_t grid = (groups + 15) / 16;
   const int64_t cap = (int64_t)num_cus() * 32;
   if (grid > cap) grid = cap;
   if (fmt == DT_E4M3)
     hipLaunchKernelGGL(token_cast128_kernel<DT_E4M3>, dim3((unsigned)grid), dim3(256), 0, s, (const uint16_t*)x,
-                       (uint8_t*)codes, scales, groups);
+                       (uint8_t*)codes, scales, rows, kblocks, mn_major);
   else if (fmt == DT_E5M2)
     hipLaunchKernelGGL(token_cast128_kernel<DT_E5M2>, dim3((unsigned)grid), dim3(256), 0, s, (const uint16_t*)x,
-                       (uint8_t*)codes, scales, groups);
+                       (uint8_t*)codes, scales, rows, kblocks, mn_major);
   else
     return set_error("unsupported fp8 format code %d", fmt);
   return check_launch("token_cast128");

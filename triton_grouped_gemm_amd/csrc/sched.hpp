@@ -126,9 +126,9 @@ TGG_DEV Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id) {
 // workgroup ids land on different XCDs (round robin over 8), so perm() hands
 // each XCD a contiguous run of P/8 tiles per sweep: neighbours in the tile order
 // (same expert weights, same activation rows) then share one XCD's L2.
-TGG_DEV int64_t sched_first_tile(int order = 0) {
+TGG_DEV int64_t sched_first_tile() {
   const int P = gridDim.x, b = blockIdx.x;
-  if (order == 0 && (P & 7) == 0) return (int64_t)(b & 7) * (P >> 3) + (b >> 3);
+  if ((P & 7) == 0) return (int64_t)(b & 7) * (P >> 3) + (b >> 3);
   return b;
 }
 

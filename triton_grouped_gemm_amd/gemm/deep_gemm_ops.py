@@ -69,7 +69,8 @@ def m_grouped_fp8_nt_contiguous(a: Tuple[torch.Tensor, torch.Tensor], b: Tuple[t
                                 use_psum_layout: bool = False) -> torch.Tensor:
     """Block-scaled FP8 grouped GEMM (reference gemm/deep_gemm_ops.py:60-100).
 
-    ``a = (codes [M_padded, K] e4m3fn, scales [M_padded, K/128] fp32)`` (1x128 recipe),
+    ``a = (codes [M_padded, K] e4m3fn, scales [M_padded, K/128] fp32)`` (1x128 recipe; any strides, no copy
+    when stored K-block-major as ``per_token_cast_to_fp8(..., scales_mn_major=True)`` returns them),
     ``b = (codes [G, N, K] e4m3fn, scales [G, ceil(N/128), K/128] fp32)`` (128x128 recipe).
     ``out[r, n] = sum_kb (sum_{k in kb} a[r,k] b[g,n,k]) * sa[r,kb] * sb[g, n//128, kb]`` with the
     scaling applied to the fp32 accumulator once per 128-deep K block; bf16 output.
@@ -94,10 +95,14 @@ def m_grouped_fp8_nt_contiguous(a: Tuple[torch.Tensor, torch.Tensor], b: Tuple[t
     _native.require_gpu(a_codes, a_scale, b_codes, b_scale, out)
     if not (a_codes.is_contiguous() and b_codes.is_contiguous() and out.is_contiguous()):
         raise ValueError("a[0], b[0] and out must be contiguous")
-    sa = a_scale.to(torch.float32).contiguous()
+    # the tuned kernel streams the activation scales one K block (= one row of a [K/128, M] array) per
+    # slab: a scale tensor that is already stored that way (strides (1, M)) is used as is
+    sa = a_scale.to(torch.float32)
+    if sa.stride() != (1, m) and kb > 1:
+        sa = sa.t().contiguous().t()
     sb = b_scale.to(torch.float32).contiguous()
     sizes, is64 = _sizes_on_device(size_per_group, a_codes.device)
     _native.call("tgg_m_grouped_gemm_fp8_block", a_codes.data_ptr(), sa.data_ptr(), b_codes.data_ptr(),
-                 sb.data_ptr(), out.data_ptr(), sizes.data_ptr(), is64, g, m, n, k, int(block_m), -1,
+                 sb.data_ptr(), out.data_ptr(), sizes.data_ptr(), is64, g, m, n, k, int(block_m), 1, -1,
                  _native.stream_of(a_codes))
     return out
