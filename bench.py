@@ -129,6 +129,8 @@ def main() -> int:
     ap.add_argument("--workload", default="bf16_m_grouped_gateup_nt", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="host-core time budget of the CPU baseline sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 1 GiB device copy (reference kernel for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the grouped-GEMM path has no cross-GPU step; run with --gpus 1", file=sys.stderr)
@@ -142,6 +144,12 @@ def main() -> int:
     torch.cuda.set_device(dev)
     fn, flops, nbytes, dtype_tag, config, cpu_sample = build_workload(args.workload, dev)
 
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, device=dev, dtype=torch.float32).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         fn()
     torch.cuda.synchronize()

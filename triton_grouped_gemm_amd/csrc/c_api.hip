@@ -11,6 +11,7 @@ namespace tgg {
 
 static thread_local char g_err[512] = "";
 static int g_force_generic = 0;
+static int g_tile_split = 1;
 
 int set_error(const char* fmt, ...) {
   va_list ap;
@@ -61,6 +62,7 @@ static int check_common(const void* A, const void* B, const void* C, const void*
 static GemmParams zero_params() {
   GemmParams p;
   memset(&p, 0, sizeof(p));
+  p.tile_split = g_tile_split;
   return p;
 }
 
@@ -240,6 +242,7 @@ int tgg_cvt_f32_to_fp8(const float* in, void* out, int64_t n, int fmt, void* str
 int tgg_set_option(const char* key, int value) {
   if (key && strcmp(key, "force_generic") == 0) { g_force_generic = value != 0; return 0; }
   if (key && strcmp(key, "variant") == 0) { set_fast_variant(value); return 0; }
+  if (key && strcmp(key, "tile_split") == 0) { g_tile_split = value != 0; return 0; }
   return set_error("unknown option '%s'", key ? key : "(null)");
 }
 

@@ -84,6 +84,7 @@ struct GemmParams {
   int N;
   int K;                  // reduction length (M-grouped); unused for K-grouped
   int grid_limit;         // >0 caps the persistent grid
+  int tile_split;         // tuned kernels: 1 = per-XCD contiguous tile ranges (see sched_walk)
 };
 
 }  // namespace tgg

@@ -173,16 +173,17 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   // 32 rows x (BN/WN) columns of 16-bit outputs, rows padded by 16 bytes.
   char* const stage_c = smem + (C::NSTAGE - 1) * C::STAGE_BYTES + wave * C::EPI_WAVE_BYTES;
 
-  int64_t tile_id = sched_first_tile();
+  const TileWalk walk = sched_walk(num_tiles, LAYOUT != LAYOUT_TN && p.tile_split);
+  int64_t tile_id = walk.first;
   Tile t;
   TileIo io;
-  if (tile_id < num_tiles) {
+  if (tile_id < walk.end) {
     t = sched_tile<C::BM, C::BN>(p, sched, tile_id);
     io = make_io(t);
 #pragma unroll
     for (int s = 0; s < C::NSTAGE - 1; ++s) issue_slab(io, s, s);
   }
-  while (tile_id < num_tiles) {
+  while (tile_id < walk.end) {
     f32x16_t acc[C::TM][C::TN];
 #pragma unroll
     for (int i = 0; i < C::TM; ++i)
@@ -234,8 +235,8 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
 
     // Request the next tile's first slabs before draining this tile's results.
     const Tile cur = t;
-    const int64_t next_id = tile_id + gridDim.x;
-    if (next_id < num_tiles) {
+    const int64_t next_id = tile_id + walk.stride;
+    if (next_id < walk.end) {
       t = sched_tile<C::BM, C::BN>(p, sched, next_id);
       io = make_io(t);
 #pragma unroll

@@ -147,11 +147,12 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
 
   char* const stage_c = smem + (C::NSTAGE - 1) * C::STAGE_BYTES + wave * C::EPI_WAVE_BYTES;
 
-  int64_t tile_id = sched_first_tile();
+  const TileWalk walk = sched_walk(num_tiles, !KGROUP && p.tile_split);
+  int64_t tile_id = walk.first;
   Tile t;
   TileIo io;
   float sbv = 0.f;
-  if (tile_id < num_tiles) {
+  if (tile_id < walk.end) {
     t = sched_tile<C::BM, C::BN>(p, sched, tile_id);
     io = make_io(t);
     sbv = load_sbv(t);
@@ -159,11 +160,11 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
 #pragma unroll
     for (int s = 0; s < C::NSTAGE - 1; ++s) issue_slab(io, s, s);
   }
-  while (tile_id < num_tiles) {
-    const int64_t next_id = tile_id + gridDim.x;
+  while (tile_id < walk.end) {
+    const int64_t next_id = tile_id + walk.stride;
     Tile nt = t;
     float sbv_next = 0.f;
-    if (next_id < num_tiles) {
+    if (next_id < walk.end) {
       nt = sched_tile<C::BM, C::BN>(p, sched, next_id);
       sbv_next = load_sbv(nt);
     }
@@ -226,7 +227,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
     __syncthreads();
 
     const Tile cur = t;
-    if (next_id < num_tiles) {
+    if (next_id < walk.end) {
       t = nt;
       io = make_io(t);
 #pragma unroll

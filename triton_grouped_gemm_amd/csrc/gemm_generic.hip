@@ -148,7 +148,8 @@ __global__ __launch_bounds__(GTHREADS) void gemm_generic_kernel(const GemmParams
   const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
   const int l32 = lane & 31, lh = lane >> 5;
 
-  for (int64_t tile_id = sched_first_tile(); tile_id < num_tiles; tile_id += gridDim.x) {
+  const TileWalk walk = sched_walk(num_tiles, !kmode);
+  for (int64_t tile_id = walk.first; tile_id < walk.end; tile_id += walk.stride) {
     const Tile t = sched_tile<GBM, GBN>(p, sm.sched, tile_id);
     // operand bases for this tile at k = 0
     const char* a_base;

@@ -122,14 +122,35 @@ TGG_DEV Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id) {
   return r;
 }
 
-// Persistent walk: workgroup b of P visits tiles it*P + perm(b).  Consecutive
-// workgroup ids land on different XCDs (round robin over 8), so perm() hands
-// each XCD a contiguous run of P/8 tiles per sweep: neighbours in the tile order
-// (same expert weights, same activation rows) then share one XCD's L2.
-TGG_DEV int64_t sched_first_tile() {
+// Persistent walk of the tile space by workgroup b of P.  Consecutive workgroup ids land on
+// different XCDs (round robin over 8), each with its own L2, so the walk is laid out per XCD:
+//   split = true   XCD x owns the contiguous tile range [x*T/8, (x+1)*T/8) and its P/8 workgroups
+//                  sweep it in runs of P/8 neighbouring tiles.  Neighbours share activation rows and
+//                  expert weights, and an expert's weights are fetched by one or two XCDs only.
+//                  Right when all tiles cost the same (M-grouped: K is fixed).
+//   split = false  every sweep hands each XCD a run of P/8 neighbouring tiles, sweeps interleaved over
+//                  the whole space.  Used when tile cost varies along the tile order (K-grouped:
+//                  cost follows the group's token count), so that every XCD sees every group.
+struct TileWalk {
+  int64_t first, end, stride;
+};
+
+TGG_DEV TileWalk sched_walk(int64_t num_tiles, bool split) {
   const int P = gridDim.x, b = blockIdx.x;
-  if ((P & 7) == 0) return (int64_t)(b & 7) * (P >> 3) + (b >> 3);
-  return b;
+  TileWalk w;
+  if ((P & 7) != 0) {
+    w.first = b; w.end = num_tiles; w.stride = P;
+  } else if (split) {
+    const int x = b & 7;
+    w.first = (num_tiles * x) / 8 + (b >> 3);
+    w.end = (num_tiles * (x + 1)) / 8;
+    w.stride = P >> 3;
+  } else {
+    w.first = (int64_t)(b & 7) * (P >> 3) + (b >> 3);
+    w.end = num_tiles;
+    w.stride = P;
+  }
+  return w;
 }
 
 }  // namespace tgg
