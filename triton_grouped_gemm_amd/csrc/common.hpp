@@ -85,6 +85,7 @@ struct GemmParams {
   int K;                  // reduction length (M-grouped); unused for K-grouped
   int grid_limit;         // >0 caps the persistent grid
   int tile_split;         // tuned kernels: 1 = per-XCD contiguous tile ranges (see sched_walk)
+  int store_nt;           // tuned kernels: 1 = non-temporal output stores
 };
 
 }  // namespace tgg

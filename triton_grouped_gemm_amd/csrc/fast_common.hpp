@@ -32,6 +32,24 @@ struct Stream {
   int64_t step;
 };
 
+// Pins a wave-uniform 64-bit value to a scalar register pair.
+TGG_DEV uint64_t uniform64(uint64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+
+// Raw buffer descriptor over [base, base + bytes), bytes clamped to [0, 2^31).
+TGG_DEV i32x4_t make_rsrc(uint64_t base, int64_t bytes) {
+  bytes = bytes < 0 ? 0 : (bytes > 0x7fffffff ? 0x7fffffff : bytes);
+  i32x4_t r;
+  r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)base);
+  r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(base >> 32) & 0xffff);  // stride 0, no swizzle
+  r[2] = __builtin_amdgcn_readfirstlane((int)bytes);
+  r[3] = 0x00020000;  // 32-bit data format
+  return r;
+}
+
 TGG_DEV i32x4_t stream_rsrc(const Stream& s, int kt) {
   const uint64_t a = s.base + (uint64_t)(kt * s.step);
   int64_t left = s.bytes - kt * s.step;

@@ -43,6 +43,12 @@ template <> struct Mma16<DT_F16> {
   }
 };
 
+// Output store; nt = streaming hint (the output is written once and not read again by this kernel).
+TGG_DEV void store_c(i32x4_t* dst, i32x4_t v, int nt) {
+  if (nt) __builtin_nontemporal_store(v, dst);
+  else *dst = v;
+}
+
 template <int BM_, int BN_, int NSTAGE_, int WM_, int WN_>
 struct FastCfg {
   static constexpr int BM = BM_, BN = BN_, NSTAGE = NSTAGE_, WM = WM_, WN = WN_;
@@ -118,55 +124,69 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
     }
   }
 
-  struct TileIo { Stream a, b; int kt_n; };
+  // Slab sequence of a tile, held in scalar registers: where the next slab of each operand starts, how
+  // many bytes may still be touched from there (everything beyond reads as zero), how many slabs exist.
+  struct TileIo {
+    uint64_t a_base, b_base;
+    int64_t a_left, b_left;
+    int kt_n, issued;
+  };
+  const int64_t a_step = A_KMAJOR ? BK * 2 : BK * a_ld;
+  const int64_t b_step = B_KMAJOR ? BK * 2 : BK * b_ld;
   auto make_io = [&](const Tile& t) {
     TileIo io;
     if (LAYOUT == LAYOUT_TN) {
       const int64_t klen = t.k1 - t.k0;
       io.kt_n = (int)((klen + BK - 1) / BK);
-      io.a.base = (uint64_t)p.A + (uint64_t)(t.k0 * a_ld + t.row0 * 2);
-      io.a.bytes = klen * a_ld - t.row0 * 2;
-      io.a.step = BK * a_ld;
-      io.b.base = (uint64_t)p.B + (uint64_t)(t.k0 * b_ld + (int64_t)t.n0 * 2);
-      io.b.bytes = klen * b_ld - (int64_t)t.n0 * 2;
-      io.b.step = BK * b_ld;
+      io.a_base = (uint64_t)p.A + (uint64_t)(t.k0 * a_ld + t.row0 * 2);
+      io.a_left = klen * a_ld - t.row0 * 2;
+      io.b_base = (uint64_t)p.B + (uint64_t)(t.k0 * b_ld + (int64_t)t.n0 * 2);
+      io.b_left = klen * b_ld - (int64_t)t.n0 * 2;
     } else {
       io.kt_n = p.K / BK;
       const int64_t rows_left = p.m_total - t.row0;
-      io.a.base = (uint64_t)p.A + (uint64_t)(t.row0 * a_ld);
-      io.a.bytes = (rows_left < C::BM ? rows_left : C::BM) * a_ld;
-      io.a.step = BK * 2;
+      io.a_base = (uint64_t)p.A + (uint64_t)(t.row0 * a_ld);
+      io.a_left = (rows_left < C::BM ? rows_left : C::BM) * a_ld;
       if (LAYOUT == LAYOUT_NT) {
         const int n_left = p.N - t.n0;
-        io.b.base = (uint64_t)p.B + (uint64_t)(((int64_t)t.g * p.N + t.n0) * b_ld);
-        io.b.bytes = (int64_t)(n_left < C::BN ? n_left : C::BN) * b_ld;
-        io.b.step = BK * 2;
+        io.b_base = (uint64_t)p.B + (uint64_t)(((int64_t)t.g * p.N + t.n0) * b_ld);
+        io.b_left = (int64_t)(n_left < C::BN ? n_left : C::BN) * b_ld;
       } else {
-        io.b.base = (uint64_t)p.B + (uint64_t)((int64_t)t.g * p.K * b_ld + (int64_t)t.n0 * 2);
-        io.b.bytes = (int64_t)p.K * b_ld - (int64_t)t.n0 * 2;
-        io.b.step = BK * b_ld;
+        io.b_base = (uint64_t)p.B + (uint64_t)((int64_t)t.g * p.K * b_ld + (int64_t)t.n0 * 2);
+        io.b_left = (int64_t)p.K * b_ld - (int64_t)t.n0 * 2;
       }
     }
+    io.a_base = uniform64(io.a_base);
+    io.b_base = uniform64(io.b_base);
+    io.a_left = (int64_t)uniform64((uint64_t)io.a_left);
+    io.b_left = (int64_t)uniform64((uint64_t)io.b_left);
+    io.kt_n = __builtin_amdgcn_readfirstlane(io.kt_n);
+    io.issued = 0;
     return io;
   };
-  // Offsets at or past this marker are outside every descriptor: such a copy fetches nothing (zeros
-  // land in LDS that nobody reads) but still takes its slot in the vmcnt bookkeeping.
-  constexpr int kNoFetch = 0x40000000;
-  auto issue_slab = [&](const TileIo& io, int kt, int buf) {
+  // Requests the tile's next slab into LDS buffer `buf`.  Past the last slab the descriptors get length
+  // zero: nothing is fetched (zeros land in a buffer nobody reads) but every wave still has the same
+  // number of copies in flight, which keeps the vmcnt arithmetic uniform.
+  auto issue_next = [&](TileIo& io, int buf) {
     const uint32_t base = smem_addr + buf * C::STAGE_BYTES;
-    const int ktc = kt < io.kt_n ? kt : 0;
-    const int dead = kt < io.kt_n ? 0 : kNoFetch;
-    const i32x4_t ra = stream_rsrc(io.a, ktc), rb = stream_rsrc(io.b, ktc);
+    const bool live = io.issued < io.kt_n;
+    const i32x4_t ra = make_rsrc(io.a_base, live ? io.a_left : 0);
+    const i32x4_t rb = make_rsrc(io.b_base, live ? io.b_left : 0);
 #pragma unroll
     for (int j = 0; j < C::NI_A / C::NWAVES; ++j) {
       const int idx = wave + j * C::NWAVES;  // wave-uniform
-      copy_b128_to_lds(ra, base + idx * 1024, a_voff + idx * OpA::RPI * (int)a_ld + dead);
+      copy_b128_to_lds(ra, base + idx * 1024, a_voff + idx * OpA::RPI * (int)a_ld);
     }
 #pragma unroll
     for (int j = 0; j < C::NI_B / C::NWAVES; ++j) {
       const int idx = wave + j * C::NWAVES;
-      copy_b128_to_lds(rb, base + C::A_BYTES + idx * 1024, b_voff + idx * OpB::RPI * (int)b_ld + dead);
+      copy_b128_to_lds(rb, base + C::A_BYTES + idx * 1024, b_voff + idx * OpB::RPI * (int)b_ld);
     }
+    io.a_base += a_step;
+    io.a_left -= a_step;
+    io.b_base += b_step;
+    io.b_left -= b_step;
+    io.issued += 1;
   };
 
   // Epilogue staging: a private region per wave inside slab buffer NSTAGE-1 (free between tiles),
@@ -175,13 +195,19 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
 
   const TileWalk walk = sched_walk(num_tiles, LAYOUT != LAYOUT_TN && p.tile_split);
   int64_t tile_id = walk.first;
-  Tile t;
-  TileIo io;
+  Tile t, nt;
+  TileIo io, nio;
   if (tile_id < walk.end) {
     t = sched_tile<C::BM, C::BN>(p, sched, tile_id);
     io = make_io(t);
 #pragma unroll
-    for (int s = 0; s < C::NSTAGE - 1; ++s) issue_slab(io, s, s);
+    for (int s = 0; s < C::NSTAGE - 1; ++s) issue_next(io, s);
+    nt = t;
+    nio = io;
+    if (tile_id + walk.stride < walk.end) {
+      nt = sched_tile<C::BM, C::BN>(p, sched, tile_id + walk.stride);
+      nio = make_io(nt);
+    }
   }
   while (tile_id < walk.end) {
     f32x16_t acc[C::TM][C::TN];
@@ -196,7 +222,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
     for (int kt = 0; kt < kt_n; ++kt) {
       wait_vmcnt<C::LPW * (C::NSTAGE - 2)>();  // this wave's share of slab kt has landed
       __syncthreads();                          // everyone's share has; everyone is done with slab kt-1
-      issue_slab(io, kt + C::NSTAGE - 1, (kt + C::NSTAGE - 1) % C::NSTAGE);
+      issue_next(io, (kt + C::NSTAGE - 1) % C::NSTAGE);
       const char* sa = smem + (kt % C::NSTAGE) * C::STAGE_BYTES;
       const char* sb = sa + C::A_BYTES;
 #pragma unroll
@@ -233,16 +259,20 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
     wait_vmcnt<0>();
     __syncthreads();  // every fragment read of this tile is done: all slab buffers are free
 
-    // Request the next tile's first slabs before draining this tile's results.
+    // Request the next tile's first slabs (its descriptors were prepared a tile ago), then look up the
+    // tile after it while those copies travel, then drain this tile's results.
     const Tile cur = t;
-    const int64_t next_id = tile_id + walk.stride;
-    if (next_id < walk.end) {
-      t = sched_tile<C::BM, C::BN>(p, sched, next_id);
-      io = make_io(t);
+    tile_id += walk.stride;
+    if (tile_id < walk.end) {
+      t = nt;
+      io = nio;
 #pragma unroll
-      for (int s = 0; s < C::NSTAGE - 1; ++s) issue_slab(io, s, s);
+      for (int s = 0; s < C::NSTAGE - 1; ++s) issue_next(io, s);
+      if (tile_id + walk.stride < walk.end) {
+        nt = sched_tile<C::BM, C::BN>(p, sched, tile_id + walk.stride);
+        nio = make_io(nt);
+      }
     }
-    tile_id = next_id;
 
     // Epilogue.  A lane owns row l32 and columns 32 j + 8 q + 4 lh + (0..3) of each 32-row block i:
     // transpose through the wave's LDS staging so that global stores are 16 bytes per lane and whole
@@ -267,7 +297,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
         const int r = it * RPIW + st_row;
         const i32x4_t v = *(const i32x4_t*)(stage_c + r * C::EPI_PITCH + st_chunk * 16);
         if (col_ok && wm0 + 32 * i + r < cur.rows)
-          *(i32x4_t*)(c_tile + ((int64_t)(32 * i + r) * p.N + st_chunk * 8) * 2) = v;
+          store_c((i32x4_t*)(c_tile + ((int64_t)(32 * i + r) * p.N + st_chunk * 8) * 2), v, p.store_nt);
       }
     }
   }

@@ -94,8 +94,9 @@ TGG_DEV Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id) {
   if (p.mode == MODE_KG || p.mode == MODE_KG_COUNT) {
     const int tiles_m = (int)((p.m_total + BM - 1) / BM);
     const int per_group = tiles_m * tiles_n;
-    r.g = (int)(tile_id / per_group);
-    const int rem = (int)(tile_id % per_group);
+    const int tid32 = (int)tile_id;
+    r.g = tid32 / per_group;
+    const int rem = tid32 % per_group;
     const int mt = rem / tiles_n;
     r.n0 = (rem % tiles_n) * BN;
     r.row0 = (int64_t)mt * BM;
@@ -105,8 +106,9 @@ TGG_DEV Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id) {
     r.k1 = r.k0 + t.rows[r.g];
     return r;
   }
-  const int mt_glob = (int)(tile_id / tiles_n);
-  r.n0 = (int)(tile_id % tiles_n) * BN;
+  const int tid32 = (int)tile_id;  // the tile space is far below 2^31; 32-bit division is much cheaper
+  const int mt_glob = tid32 / tiles_n;
+  r.n0 = (tid32 % tiles_n) * BN;
   int lo = 0, hi = p.G;  // last g with tile0[g] <= mt_glob
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
