@@ -10,8 +10,13 @@
 //     VGPR staging.  Anything outside an operand (rows past the end of A, tokens past the end of
 //     a group's range) reads as zero through the buffer descriptor's bounds check, so ragged
 //     groups and token tails need no separate code path.
-//   * NSTAGE slabs rotate through LDS with one workgroup barrier per slab; the first slabs of the
-//     next tile are requested before the current tile's results are drained.
+//   * Two slab buffers alternate in LDS with one workgroup barrier per slab.  The slabs of all of a
+//     workgroup's tiles form one uninterrupted stream: the copies run two slabs ahead of the
+//     multiplies across tile boundaries, and the fragment reads run one K step ahead across the
+//     barrier, so neither the barrier nor the LDS latency behind it leaves the matrix pipe idle.
+//   * A slab's copy instructions are issued one per two multiplies rather than back to back: the
+//     address unit takes 16 cycles per copy and has a short queue, and a wave blocked on that queue
+//     cannot issue its multiplies.
 //   * LDS is XOR-swizzled at 16-byte granularity.  The direct-to-LDS copy is lane-linear on the
 //     LDS side, so the swizzle is applied to the global address each lane fetches from.
 //   * K-contiguous operands are read back as 16-byte MFMA fragments (ds_read_b128); operands whose
@@ -19,8 +24,8 @@
 //     every lane 4 consecutive K values of one column.
 //   * Each wave owns a (BM/WM) x (BN/WN) block of 32x32x16 MFMA tiles, issued with the B operand as
 //     srcA and the A operand as srcB, so a lane ends up with 4 consecutive output columns of one
-//     row; results are transposed through a per-wave LDS staging area and leave as 16-byte stores
-//     covering whole 128-byte row segments.
+//     row; results are transposed 32x32 block by block through a small per-wave LDS staging area
+//     (separate from the slab buffers, so the copy stream keeps running) and leave as 16-byte stores.
 #include "fast_common.hpp"
 #include "launch.hpp"
 
@@ -49,23 +54,23 @@ TGG_DEV void store_c(i32x4_t* dst, i32x4_t v, int nt) {
   else *dst = v;
 }
 
-template <int BM_, int BN_, int NSTAGE_, int WM_, int WN_>
+template <int BM_, int BN_, int WM_, int WN_>
 struct FastCfg {
-  static constexpr int BM = BM_, BN = BN_, NSTAGE = NSTAGE_, WM = WM_, WN = WN_;
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
   static constexpr int NWAVES = WM * WN;
   static constexpr int THREADS = NWAVES * 64;
   static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   static constexpr int NI_A = A_BYTES / 1024, NI_B = B_BYTES / 1024;
-  static constexpr int LPW = (NI_A + NI_B) / NWAVES;  // copies per wave per slab
   static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-  static constexpr int EPI_PITCH = (BN / WN) * 2 + 16;  // staged output row pitch in bytes
+  static constexpr int EPI_PITCH = 32 * 2 + 16;  // staged 32x32 output block: row pitch in bytes
   static constexpr int EPI_WAVE_BYTES = 32 * EPI_PITCH;
-  static constexpr int SMEM_BYTES = NSTAGE * STAGE_BYTES + (int)sizeof(SchedTableT<kFastMaxGroups>);
+  static constexpr int SCHED_OFF = 2 * STAGE_BYTES;
+  static constexpr int EPI_OFF = SCHED_OFF + (((int)sizeof(SchedTableT<kFastMaxGroups>) + 255) & ~255);
+  static constexpr int SMEM_BYTES = EPI_OFF + NWAVES * EPI_WAVE_BYTES;
   static_assert(NI_A % NWAVES == 0 && NI_B % NWAVES == 0, "copies must divide evenly over waves");
   static_assert(NWAVES % 4 == 0, "a wave keeps one swizzle pattern for all its copies");
-  static_assert(LPW * (NSTAGE - 1) < 64, "vmcnt range");
-  static_assert(NWAVES * EPI_WAVE_BYTES <= STAGE_BYTES, "epilogue staging must fit in one slab buffer");
+  static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
 };
 
 template <class C, int DT, int LAYOUT>
@@ -76,7 +81,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   typedef Operand<C::BN, B_KMAJOR> OpB;
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::NSTAGE * C::STAGE_BYTES);
+  auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::SCHED_OFF);
   sched_init<C::BM>(p, sched);
   const int64_t num_tiles = sched_num_tiles<C::BM, C::BN>(p, sched);
 
@@ -123,6 +128,32 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
       b_rd[j2] = ((blk >> 1) * 8 + e) * (C::BN * 2) + chunk * 16 + (c & 1) * 8;
     }
   }
+  // MFMA fragments of K step ks of the slab at sa (A part) / sb (B part)
+  auto load_frags = [&](const char* sa, int ks, i32x4_t (&fa)[C::TM], i32x4_t (&fb)[C::TN]) {
+    const char* sb = sa + C::A_BYTES;
+#pragma unroll
+    for (int i = 0; i < C::TM; ++i) {
+      if (A_KMAJOR) {
+        fa[i] = *(const i32x4_t*)(sa + a_rd[ks] + i * 32 * 128);
+      } else {
+        const char* q = sa + a_rd[i] + ks * 16 * (C::BM * 2);
+        const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)q);
+        const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)(q + 4 * (C::BM * 2)));
+        fa[i] = __builtin_bit_cast(i32x4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j) {
+      if (B_KMAJOR) {
+        fb[j] = *(const i32x4_t*)(sb + b_rd[ks] + j * 32 * 128);
+      } else {
+        const char* q = sb + b_rd[j] + ks * 16 * (C::BN * 2);
+        const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)q);
+        const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)(q + 4 * (C::BN * 2)));
+        fb[j] = __builtin_bit_cast(i32x4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    }
+  };
 
   // Slab sequence of a tile, held in scalar registers: where the next slab of each operand starts, how
   // many bytes may still be touched from there (everything beyond reads as zero), how many slabs exist.
@@ -133,17 +164,19 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   };
   const int64_t a_step = A_KMAJOR ? BK * 2 : BK * a_ld;
   const int64_t b_step = B_KMAJOR ? BK * 2 : BK * b_ld;
+  auto slabs_of = [&](const Tile& t) -> int {
+    return LAYOUT == LAYOUT_TN ? (int)((t.k1 - t.k0 + BK - 1) / BK) : p.K / BK;
+  };
   auto make_io = [&](const Tile& t) {
     TileIo io;
+    io.kt_n = slabs_of(t);
     if (LAYOUT == LAYOUT_TN) {
       const int64_t klen = t.k1 - t.k0;
-      io.kt_n = (int)((klen + BK - 1) / BK);
       io.a_base = (uint64_t)p.A + (uint64_t)(t.k0 * a_ld + t.row0 * 2);
       io.a_left = klen * a_ld - t.row0 * 2;
       io.b_base = (uint64_t)p.B + (uint64_t)(t.k0 * b_ld + (int64_t)t.n0 * 2);
       io.b_left = klen * b_ld - (int64_t)t.n0 * 2;
     } else {
-      io.kt_n = p.K / BK;
       const int64_t rows_left = p.m_total - t.row0;
       io.a_base = (uint64_t)p.A + (uint64_t)(t.row0 * a_ld);
       io.a_left = (rows_left < C::BM ? rows_left : C::BM) * a_ld;
@@ -164,52 +197,92 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
     io.issued = 0;
     return io;
   };
-  // Requests the tile's next slab into LDS buffer `buf`.  Past the last slab the descriptors get length
-  // zero: nothing is fetched (zeros land in a buffer nobody reads) but every wave still has the same
-  // number of copies in flight, which keeps the vmcnt arithmetic uniform.
-  auto issue_next = [&](TileIo& io, int buf) {
-    const uint32_t base = smem_addr + buf * C::STAGE_BYTES;
-    const bool live = io.issued < io.kt_n;
-    const i32x4_t ra = make_rsrc(io.a_base, live ? io.a_left : 0);
-    const i32x4_t rb = make_rsrc(io.b_base, live ? io.b_left : 0);
-#pragma unroll
-    for (int j = 0; j < C::NI_A / C::NWAVES; ++j) {
-      const int idx = wave + j * C::NWAVES;  // wave-uniform
-      copy_b128_to_lds(ra, base + idx * 1024, a_voff + idx * OpA::RPI * (int)a_ld);
+
+  // The copy stream.  Slabs of all of this workgroup's tiles form one sequence (tiles without slabs,
+  // i.e. empty K-grouped segments, contribute nothing); slab q of the sequence lives in LDS buffer
+  // q % 2.  `feed` is the tile whose slabs are being requested, normally one tile ahead of the tile
+  // being multiplied.  Once the sequence is exhausted the descriptors get length zero: nothing is
+  // fetched, but every wave still issues the same number of copies, which keeps the waits uniform.
+  const TileWalk walk = sched_walk(num_tiles, LAYOUT != LAYOUT_TN && p.tile_split);
+  TileIo feed;
+  int64_t feed_id;
+  auto feed_seek = [&](int64_t id) {
+    feed.kt_n = 0;
+    feed.issued = 0;
+    feed.a_base = feed.b_base = (uint64_t)p.A;
+    feed.a_left = feed.b_left = 0;
+    for (; id < walk.end; id += walk.stride) {
+      const Tile tt = sched_tile<C::BM, C::BN>(p, sched, id);
+      if (slabs_of(tt) > 0) {
+        feed = make_io(tt);
+        break;
+      }
     }
-#pragma unroll
-    for (int j = 0; j < C::NI_B / C::NWAVES; ++j) {
-      const int idx = wave + j * C::NWAVES;
-      copy_b128_to_lds(rb, base + C::A_BYTES + idx * 1024, b_voff + idx * OpB::RPI * (int)b_ld);
+    feed_id = id;
+  };
+  // One slab's copies are requested in two halves, interleaved with multiplies (see the pipeline below):
+  // begin_slab fixes the descriptors and moves the feed on, copy_k issues this wave's k-th copy.
+  struct SlabCopy {
+    i32x4_t ra, rb;
+    uint32_t base;
+  };
+  constexpr int CA = C::NI_A / C::NWAVES, CB = C::NI_B / C::NWAVES, NC = CA + CB;
+  constexpr int SP = (C::TM * C::TN) / (NC / 2);  // multiplies between two copies
+  static_assert(NC % 2 == 0 && SP >= 1, "a slab's copies are spread over the multiplies of two K steps");
+  auto begin_slab = [&](int buf) {
+    SlabCopy sc;
+    const bool live = feed.issued < feed.kt_n;
+    sc.ra = make_rsrc(feed.a_base, live ? feed.a_left : 0);
+    sc.rb = make_rsrc(feed.b_base, live ? feed.b_left : 0);
+    sc.base = smem_addr + buf * C::STAGE_BYTES;
+    feed.a_base += a_step;
+    feed.a_left -= a_step;
+    feed.b_base += b_step;
+    feed.b_left -= b_step;
+    feed.issued += 1;
+    if (live && feed.issued >= feed.kt_n) feed_seek(feed_id + walk.stride);
+    return sc;
+  };
+  auto copy_k = [&](const SlabCopy& sc, int k) {
+    if (k < CA) {
+      const int idx = wave + k * C::NWAVES;  // wave-uniform
+      copy_b128_to_lds(sc.ra, sc.base + idx * 1024, a_voff + idx * OpA::RPI * (int)a_ld);
+    } else {
+      const int idx = wave + (k - CA) * C::NWAVES;
+      copy_b128_to_lds(sc.rb, sc.base + C::A_BYTES + idx * 1024, b_voff + idx * OpB::RPI * (int)b_ld);
     }
-    io.a_base += a_step;
-    io.a_left -= a_step;
-    io.b_base += b_step;
-    io.b_left -= b_step;
-    io.issued += 1;
   };
 
-  // Epilogue staging: a private region per wave inside slab buffer NSTAGE-1 (free between tiles),
-  // 32 rows x (BN/WN) columns of 16-bit outputs, rows padded by 16 bytes.
-  char* const stage_c = smem + (C::NSTAGE - 1) * C::STAGE_BYTES + wave * C::EPI_WAVE_BYTES;
+  // Epilogue staging: a private 32x32 block of 16-bit outputs per wave, rows padded by 16 bytes.
+  char* const stage_c = smem + C::EPI_OFF + wave * C::EPI_WAVE_BYTES;
 
-  const TileWalk walk = sched_walk(num_tiles, LAYOUT != LAYOUT_TN && p.tile_split);
-  int64_t tile_id = walk.first;
-  Tile t, nt;
-  TileIo io, nio;
-  if (tile_id < walk.end) {
-    t = sched_tile<C::BM, C::BN>(p, sched, tile_id);
-    io = make_io(t);
+  // Software pipeline.  Per slab r (4 K steps of 16):
+  //   steps 0..2  read the fragments of the following step while multiplying the current one;
+  //   step 3      wait for this wave's share of slab r+1, workgroup barrier (now slab r+1 is complete and
+  //               nobody reads slab r any more: its last fragments are already in registers), read step 0
+  //               of slab r+1, and only then multiply step 3.
+  // The copies of slab r+2 (into slab r's buffer) are issued one per two multiplies during step 3 and
+  // the following step 0: the texture-address unit takes 16 cycles per copy instruction and its queue
+  // is short, so a wave that issues its copies back to back sits blocked behind the other waves'
+  // copies with its multiplies queued up behind them.  Tile boundaries do not interrupt the stream.
+  feed_seek(walk.first);
+  {
+    const SlabCopy s0 = begin_slab(0);
 #pragma unroll
-    for (int s = 0; s < C::NSTAGE - 1; ++s) issue_next(io, s);
-    nt = t;
-    nio = io;
-    if (tile_id + walk.stride < walk.end) {
-      nt = sched_tile<C::BM, C::BN>(p, sched, tile_id + walk.stride);
-      nio = make_io(nt);
-    }
+    for (int k = 0; k < NC; ++k) copy_k(s0, k);
   }
-  while (tile_id < walk.end) {
+  wait_vmcnt<0>();
+  __syncthreads();
+  SlabCopy sc = begin_slab(1);
+#pragma unroll
+  for (int k = 0; k < NC / 2; ++k) copy_k(sc, k);
+  i32x4_t fa0[C::TM], fb0[C::TN], fa1[C::TM], fb1[C::TN];
+  load_frags(smem, 0, fa0, fb0);
+  int ring = 0;
+
+  for (int64_t tile_id = walk.first; tile_id < walk.end; tile_id += walk.stride) {
+    const Tile cur = sched_tile<C::BM, C::BN>(p, sched, tile_id);
+    const int kt_n = __builtin_amdgcn_readfirstlane(slabs_of(cur));
     f32x16_t acc[C::TM][C::TN];
 #pragma unroll
     for (int i = 0; i < C::TM; ++i)
@@ -218,89 +291,71 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    const int kt_n = io.kt_n;
-    for (int kt = 0; kt < kt_n; ++kt) {
-      wait_vmcnt<C::LPW * (C::NSTAGE - 2)>();  // this wave's share of slab kt has landed
-      __syncthreads();                          // everyone's share has; everyone is done with slab kt-1
-      issue_next(io, (kt + C::NSTAGE - 1) % C::NSTAGE);
-      const char* sa = smem + (kt % C::NSTAGE) * C::STAGE_BYTES;
-      const char* sb = sa + C::A_BYTES;
+    // One K step: multiply (fa, fb); right after the first multiply, read the fragments of K step ks_next
+    // of the slab at s_next into (fna, fnb); copies [k0, k0 + NC/2) of `sc` are issued one per SP
+    // multiplies when k0 >= 0.
+    auto step = [&](const i32x4_t (&fa)[C::TM], const i32x4_t (&fb)[C::TN], const char* s_next, int ks_next,
+                    i32x4_t (&fna)[C::TM], i32x4_t (&fnb)[C::TN], int k0) {
 #pragma unroll
-      for (int ks = 0; ks < BK / 16; ++ks) {
-        i32x4_t fa[C::TM], fb[C::TN];
-#pragma unroll
-        for (int i = 0; i < C::TM; ++i) {
-          if (A_KMAJOR) {
-            fa[i] = *(const i32x4_t*)(sa + a_rd[ks] + i * 32 * 128);
-          } else {
-            const char* q = sa + a_rd[i] + ks * 16 * (C::BM * 2);
-            const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)q);
-            const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)(q + 4 * (C::BM * 2)));
-            fa[i] = __builtin_bit_cast(i32x4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-          }
-        }
+      for (int i = 0; i < C::TM; ++i)
 #pragma unroll
         for (int j = 0; j < C::TN; ++j) {
-          if (B_KMAJOR) {
-            fb[j] = *(const i32x4_t*)(sb + b_rd[ks] + j * 32 * 128);
-          } else {
-            const char* q = sb + b_rd[j] + ks * 16 * (C::BN * 2);
-            const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)q);
-            const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)(q + 4 * (C::BN * 2)));
-            fb[j] = __builtin_bit_cast(i32x4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+          acc[i][j] = Mma16<DT>::run(fb[j], fa[i], acc[i][j]);
+          const int n = i * C::TN + j;
+          if (n == 0) {
+            __builtin_amdgcn_sched_barrier(0);
+            load_frags(s_next, ks_next, fna, fnb);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          if (k0 >= 0 && (n + 1) % SP == 0 && (n + 1) / SP <= NC / 2) {
+            __builtin_amdgcn_sched_barrier(0);
+            copy_k(sc, k0 + (n + 1) / SP - 1);
+            __builtin_amdgcn_sched_barrier(0);
           }
         }
-#pragma unroll
-        for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-          for (int j = 0; j < C::TN; ++j) acc[i][j] = Mma16<DT>::run(fb[j], fa[i], acc[i][j]);
-      }
-    }
-    wait_vmcnt<0>();
-    __syncthreads();  // every fragment read of this tile is done: all slab buffers are free
+      __builtin_amdgcn_sched_barrier(0);
+    };
 
-    // Request the next tile's first slabs (its descriptors were prepared a tile ago), then look up the
-    // tile after it while those copies travel, then drain this tile's results.
-    const Tile cur = t;
-    tile_id += walk.stride;
-    if (tile_id < walk.end) {
-      t = nt;
-      io = nio;
-#pragma unroll
-      for (int s = 0; s < C::NSTAGE - 1; ++s) issue_next(io, s);
-      if (tile_id + walk.stride < walk.end) {
-        nt = sched_tile<C::BM, C::BN>(p, sched, tile_id + walk.stride);
-        nio = make_io(nt);
-      }
+    for (int kt = 0; kt < kt_n; ++kt) {
+      const char* sa = smem + (ring & 1) * C::STAGE_BYTES;
+      const char* sn = smem + ((ring + 1) & 1) * C::STAGE_BYTES;
+      step(fa0, fb0, sa, 1, fa1, fb1, NC / 2);
+      step(fa1, fb1, sa, 2, fa0, fb0, -1);
+      step(fa0, fb0, sa, 3, fa1, fb1, -1);
+      const SlabCopy sc_next = begin_slab(ring & 1);  // scalar work only: overlaps the multiplies in flight
+      wait_vmcnt<0>();
+      __syncthreads();
+      sc = sc_next;
+      step(fa1, fb1, sn, 0, fa0, fb0, 0);
+      ++ring;
     }
 
     // Epilogue.  A lane owns row l32 and columns 32 j + 8 q + 4 lh + (0..3) of each 32-row block i:
-    // transpose through the wave's LDS staging so that global stores are 16 bytes per lane and whole
-    // 128-byte (or longer) row segments per instruction.
-    constexpr int WCOLS = C::BN / C::WN;  // columns owned by this wave
-    constexpr int CPRW = WCOLS / 8;       // 16-byte chunks per staged row
-    constexpr int RPIW = 64 / CPRW;       // rows covered by one wave-wide read
+    // transpose each 32x32 block through the wave's LDS staging so that global stores are 16 bytes per
+    // lane and 64-byte row segments, two neighbouring rows' worth per 128 bytes of a wave's store.
     const int64_t c_row0 = (LAYOUT == LAYOUT_TN) ? ((int64_t)cur.g * p.m_total + cur.row0) : cur.row0;
     char* const c_tile = (char*)p.C + ((c_row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2;
-    const int st_row = lane / CPRW, st_chunk = lane % CPRW;
-    const bool col_ok = cur.n0 + wn0 + st_chunk * 8 < p.N;
+    const int st_row = lane >> 2, st_chunk = lane & 3;
 #pragma unroll
     for (int i = 0; i < C::TM; ++i) {
 #pragma unroll
-      for (int j = 0; j < C::TN; ++j)
+      for (int j = 0; j < C::TN; ++j) {
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          *(uint2*)(stage_c + l32 * C::EPI_PITCH + (32 * j + 8 * q + 4 * lh) * 2) =
+          *(uint2*)(stage_c + l32 * C::EPI_PITCH + (8 * q + 4 * lh) * 2) =
               pack4<DT>(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+        const bool col_ok = cur.n0 + wn0 + 32 * j + st_chunk * 8 < p.N;
 #pragma unroll
-      for (int it = 0; it < 32 / RPIW; ++it) {
-        const int r = it * RPIW + st_row;
-        const i32x4_t v = *(const i32x4_t*)(stage_c + r * C::EPI_PITCH + st_chunk * 16);
-        if (col_ok && wm0 + 32 * i + r < cur.rows)
-          store_c((i32x4_t*)(c_tile + ((int64_t)(32 * i + r) * p.N + st_chunk * 8) * 2), v, p.store_nt);
+        for (int it = 0; it < 2; ++it) {
+          const int r = it * 16 + st_row;
+          const i32x4_t v = *(const i32x4_t*)(stage_c + r * C::EPI_PITCH + st_chunk * 16);
+          if (col_ok && wm0 + 32 * i + r < cur.rows)
+            store_c((i32x4_t*)(c_tile + ((int64_t)(32 * i + r) * p.N + 32 * j + st_chunk * 8) * 2), v, p.store_nt);
+        }
       }
     }
   }
+  wait_vmcnt<0>();  // the trailing zero-length copies still write LDS: let them finish before the wave ends
 }
 
 template <class C, int DT, int LAYOUT>
@@ -326,11 +381,8 @@ template <int DT, int LAYOUT>
 int launch_variant(const GemmParams& p, hipStream_t s) {
   switch (g_variant) {
     default:
-    case 0: return launch_cfg<FastCfg<256, 256, 2, 2, 4>, DT, LAYOUT>(p, s);
-    case 1: return launch_cfg<FastCfg<256, 128, 3, 4, 2>, DT, LAYOUT>(p, s);
-    case 2: return launch_cfg<FastCfg<256, 128, 3, 2, 4>, DT, LAYOUT>(p, s);
-    case 3: return launch_cfg<FastCfg<128, 256, 3, 2, 4>, DT, LAYOUT>(p, s);
-    case 4: return launch_cfg<FastCfg<128, 128, 4, 2, 2>, DT, LAYOUT>(p, s);
+    case 0: return launch_cfg<FastCfg<256, 256, 2, 4>, DT, LAYOUT>(p, s);
+    case 1: return launch_cfg<FastCfg<256, 128, 2, 4>, DT, LAYOUT>(p, s);
   }
 }
 
