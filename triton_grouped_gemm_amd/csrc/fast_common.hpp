@@ -24,14 +24,6 @@ TGG_DEV void copy_b128_to_lds(i32x4_t rsrc, uint32_t lds_addr, int voff) {
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
 }
 
-// A run of slabs of one operand: slab kt starts at base + kt * step and may touch `bytes - kt * step`
-// bytes from there (everything beyond reads as zero).  All fields are wave-uniform.
-struct Stream {
-  uint64_t base;
-  int64_t bytes;
-  int64_t step;
-};
-
 // Pins a wave-uniform 64-bit value to a scalar register pair.
 TGG_DEV uint64_t uniform64(uint64_t v) {
   const uint32_t lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)v);
@@ -47,18 +39,6 @@ TGG_DEV i32x4_t make_rsrc(uint64_t base, int64_t bytes) {
   r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(base >> 32) & 0xffff);  // stride 0, no swizzle
   r[2] = __builtin_amdgcn_readfirstlane((int)bytes);
   r[3] = 0x00020000;  // 32-bit data format
-  return r;
-}
-
-TGG_DEV i32x4_t stream_rsrc(const Stream& s, int kt) {
-  const uint64_t a = s.base + (uint64_t)(kt * s.step);
-  int64_t left = s.bytes - kt * s.step;
-  left = left < 0 ? 0 : (left > 0x7fffffff ? 0x7fffffff : left);
-  i32x4_t r;  // readfirstlane pins the descriptor to scalar registers
-  r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
-  r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32) & 0xffff);  // stride 0, no swizzle
-  r[2] = __builtin_amdgcn_readfirstlane((int)left);
-  r[3] = 0x00020000;  // raw buffer, 32-bit data format
   return r;
 }
 

@@ -1,8 +1,9 @@
 // Tuned FP8 (OCP e4m3fn / e5m2) grouped GEMM kernels for gfx950, K-contiguous operands.
 //
-// Same skeleton as the 16-bit kernels (persistent grouped tiles, direct-to-LDS slabs, swizzled
-// LDS, staged epilogue); a slab is 128 bytes = 128 K values of every row, i.e. exactly one
-// 128-wide scale block.  The contraction runs on v_mfma_f32_32x32x64_f8f6f4.
+// Same skeleton as the 16-bit kernels (persistent grouped tiles, one continuous direct-to-LDS slab
+// stream across tiles, swizzled LDS, copies interleaved with multiplies, staged epilogue); a slab is
+// 128 bytes = 128 K values of every row, i.e. exactly one 128-wide scale block.  The contraction runs
+// on v_mfma_f32_32x32x64_f8f6f4.
 //
 //   EPI_BLOCK    out[r,n] = sum_kb (sum_{k in kb} a[r,k] b[g,n,k]) * sa[kb,r] * sb[g,n/128,kb]
 //                Every slab is contracted into a fresh partial accumulator that is then folded into
@@ -27,19 +28,9 @@ TGG_DEV void copy_b32_to_lds(i32x4_t rsrc, uint32_t lds_addr, int voff) {
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
 }
 
-TGG_DEV i32x4_t raw_rsrc(uint64_t a, int64_t bytes) {
-  bytes = bytes < 0 ? 0 : (bytes > 0x7fffffff ? 0x7fffffff : bytes);
-  i32x4_t r;
-  r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)a);
-  r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(a >> 32) & 0xffff);
-  r[2] = __builtin_amdgcn_readfirstlane((int)bytes);
-  r[3] = 0x00020000;
-  return r;
-}
-
-template <int BM_, int BN_, int NSTAGE_, int WM_, int WN_>
+template <int BM_, int BN_, int WM_, int WN_>
 struct Fp8Cfg {
-  static constexpr int BM = BM_, BN = BN_, NSTAGE = NSTAGE_, WM = WM_, WN = WN_;
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
   static constexpr int NWAVES = WM * WN;
   static constexpr int THREADS = NWAVES * 64;
   static constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128;
@@ -47,13 +38,16 @@ struct Fp8Cfg {
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + SA_BYTES;
   static constexpr int NI_A = A_BYTES / 1024, NI_B = B_BYTES / 1024;
   static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-  static constexpr int EPI_PITCH = (BN / WN) * 2 + 16;
+  static constexpr int EPI_PITCH = 32 * 2 + 16;  // staged 32x32 output block: row pitch in bytes
   static constexpr int EPI_WAVE_BYTES = 32 * EPI_PITCH;
-  static constexpr int SMEM_BYTES = NSTAGE * STAGE_BYTES + (int)sizeof(SchedTableT<kFastMaxGroups>);
+  static constexpr int SCHED_OFF = 2 * STAGE_BYTES;
+  static constexpr int EPI_OFF = SCHED_OFF + (((int)sizeof(SchedTableT<kFastMaxGroups>) + 255) & ~255);
+  static constexpr int SMEM_BYTES = EPI_OFF + NWAVES * EPI_WAVE_BYTES;
   static_assert(NI_A % NWAVES == 0 && NI_B % NWAVES == 0, "copies must divide evenly over waves");
   static_assert(NWAVES % 2 == 0 && BM / 64 <= NWAVES, "scale copies: one per wave");
   static_assert((BN / WN) <= 128, "a wave's columns must share one 128-wide weight scale block");
-  static_assert(NWAVES * EPI_WAVE_BYTES <= A_BYTES + B_BYTES, "epilogue staging must fit in one slab buffer");
+  static_assert(TN == 2 && TM % 2 == 0, "the cell schedule below alternates two B fragments and two A buffers");
+  static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
 };
 
 // FA / FB: 0 = e4m3fn, 1 = e5m2 (the cbsz / blgp format codes of the f8f6f4 MFMA).
@@ -61,11 +55,10 @@ template <class C, int FA, int FB, int EPI, int OUT, bool KGROUP>
 __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p) {
   typedef Operand<C::BM, true> OpA;
   typedef Operand<C::BN, true> OpB;
-  constexpr int LPW = (C::NI_A + C::NI_B) / C::NWAVES + (EPI == EPI_BLOCK ? 1 : 0);  // copies per wave per slab
-  static_assert(LPW * (C::NSTAGE - 1) < 64, "vmcnt range");
+  constexpr bool BLOCK = EPI == EPI_BLOCK;
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::NSTAGE * C::STAGE_BYTES);
+  auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::SCHED_OFF);
   sched_init<C::BM>(p, sched);
   const int64_t num_tiles = sched_num_tiles<C::BM, C::BN>(p, sched);
 
@@ -89,83 +82,154 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
   for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
     for (int h = 0; h < 2; ++h) rd[ks][h] = l32 * 128 + (((4 * ks + 2 * lh + h) ^ fsw) << 4);
+  // both K steps of one 32-row block starting at LDS address q
+  auto load_frag = [&](const char* q, i32x8_t (&f)[2]) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const i32x4_t lo = *(const i32x4_t*)(q + rd[ks][0]);
+      const i32x4_t hi = *(const i32x4_t*)(q + rd[ks][1]);
+      f[ks] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+  };
 
-  struct TileIo { Stream a, b; uint64_t sa_base; int sa_bytes; int kt_n; };
+  // Slab sequence of a tile in scalar registers (see gemm_fast.hip): next slab's start and remaining bytes
+  // of A, B and (block scaling) of the tile rows' activation scales, which are stored [K/128, m_total].
+  struct TileIo {
+    uint64_t a_base, b_base, s_base;
+    int64_t a_left, b_left;
+    int s_bytes, kt_n, issued;
+  };
+  auto slabs_of = [&](const Tile& t) -> int { return KGROUP ? (int)((t.k1 - t.k0 + BKB - 1) / BKB) : p.K / BKB; };
   auto make_io = [&](const Tile& t) {
     TileIo io;
     const int64_t k0 = KGROUP ? t.k0 : 0;
-    io.kt_n = KGROUP ? (int)((t.k1 - t.k0 + BKB - 1) / BKB) : p.K / BKB;
+    io.kt_n = __builtin_amdgcn_readfirstlane(slabs_of(t));
     const int64_t rows_left = p.m_total - t.row0;
     const int a_rows = (int)(rows_left < C::BM ? rows_left : C::BM);
     const int n_left = p.N - t.n0;
-    io.a.base = (uint64_t)p.A + (uint64_t)(t.row0 * ld + k0);
-    io.a.bytes = (int64_t)a_rows * ld - k0;
-    io.a.step = BKB;
-    io.b.base = (uint64_t)p.B + (uint64_t)((KGROUP ? (int64_t)t.n0 : ((int64_t)t.g * p.N + t.n0)) * ld + k0);
-    io.b.bytes = (int64_t)(n_left < C::BN ? n_left : C::BN) * ld - k0;
-    io.b.step = BKB;
-    io.sa_base = 0;
-    io.sa_bytes = 0;
-    if (EPI == EPI_BLOCK) {
-      io.sa_base = (uint64_t)(p.sa + t.row0);   // [kblocks, m_total]: row kb starts m_total floats further
-      io.sa_bytes = a_rows * 4;
-    }
+    io.a_base = uniform64((uint64_t)p.A + (uint64_t)(t.row0 * ld + k0));
+    io.a_left = (int64_t)uniform64((uint64_t)((int64_t)a_rows * ld - k0));
+    io.b_base = uniform64((uint64_t)p.B + (uint64_t)((KGROUP ? (int64_t)t.n0 : ((int64_t)t.g * p.N + t.n0)) * ld + k0));
+    io.b_left = (int64_t)uniform64((uint64_t)((int64_t)(n_left < C::BN ? n_left : C::BN) * ld - k0));
+    io.s_base = BLOCK ? uniform64((uint64_t)(p.sa + t.row0)) : 0;
+    io.s_bytes = BLOCK ? __builtin_amdgcn_readfirstlane(a_rows * 4) : 0;
+    io.issued = 0;
     return io;
   };
   // Weight scales of this wave's column block for every slab of a tile: lane kb holds block kb.
   // This is an ordinary vector load, so the compiler waits for *all* outstanding vector memory
   // traffic at its first use; it is therefore fetched one tile ahead and first touched right after
-  // the end-of-tile drain, where nothing is in flight anyway.
+  // a point where this wave has waited for everything anyway.
   auto load_sbv = [&](const Tile& t) {
     const int64_t idx = ((int64_t)t.g * nblocks + ((t.n0 + wn0) >> 7)) * kblocks;
-    return (EPI == EPI_BLOCK && lane < kblocks) ? p.sb[idx + lane] : 0.f;
+    return (BLOCK && lane < kblocks) ? p.sb[idx + lane] : 0.f;
+  };
+
+  // The copy stream (see gemm_fast.hip): slab q of the workgroup's whole slab sequence lives in buffer q % 2.
+  // Interleaved sweeps: with 1-byte operands an expert's weight panel set is twice as deep in K for the same
+  // bytes, and letting all XCDs share the experts in flight through the memory-side cache measured ~3% faster
+  // (and half the L2 fill traffic) than giving each XCD its own contiguous range of tiles.
+  const TileWalk walk = sched_walk(num_tiles, false);
+  TileIo feed;
+  int64_t feed_id;
+  auto feed_seek = [&](int64_t id) {
+    feed.kt_n = 0;
+    feed.issued = 0;
+    feed.a_base = feed.b_base = feed.s_base = (uint64_t)p.A;
+    feed.a_left = feed.b_left = 0;
+    feed.s_bytes = 0;
+    for (; id < walk.end; id += walk.stride) {
+      const Tile tt = sched_tile<C::BM, C::BN>(p, sched, id);
+      if (slabs_of(tt) > 0) {
+        feed = make_io(tt);
+        break;
+      }
+    }
+    feed_id = id;
+  };
+  struct SlabCopy {
+    i32x4_t ra, rb, rs;
+    uint32_t base;
+  };
+  constexpr int CA = C::NI_A / C::NWAVES, CB = C::NI_B / C::NWAVES, CS = BLOCK ? 1 : 0, NC = CS + CA + CB;
+  auto begin_slab = [&](int buf) {
+    SlabCopy sc;
+    const bool live = feed.issued < feed.kt_n;
+    sc.ra = make_rsrc(feed.a_base, live ? feed.a_left : 0);
+    sc.rb = make_rsrc(feed.b_base, live ? feed.b_left : 0);
+    sc.rs = make_rsrc(feed.s_base, live ? feed.s_bytes : 0);
+    sc.base = smem_addr + buf * C::STAGE_BYTES;
+    feed.a_base += BKB;
+    feed.a_left -= BKB;
+    feed.b_base += BKB;
+    feed.b_left -= BKB;
+    feed.s_base += (uint64_t)p.m_total * 4;
+    feed.issued += 1;
+    if (live && feed.issued >= feed.kt_n) feed_seek(feed_id + walk.stride);
+    return sc;
   };
   constexpr int kNoFetch = 0x40000000;
-  auto issue_slab = [&](const TileIo& io, int kt, int buf) {
-    const uint32_t base = smem_addr + buf * C::STAGE_BYTES;
-    const int ktc = kt < io.kt_n ? kt : 0;
-    const int dead = kt < io.kt_n ? 0 : kNoFetch;
-    const i32x4_t ra = stream_rsrc(io.a, ktc), rb = stream_rsrc(io.b, ktc);
-#pragma unroll
-    for (int j = 0; j < C::NI_A / C::NWAVES; ++j) {
-      const int idx = wave + j * C::NWAVES;
-      copy_b128_to_lds(ra, base + idx * 1024, a_voff + idx * OpA::RPI * (int)ld + dead);
-    }
-#pragma unroll
-    for (int j = 0; j < C::NI_B / C::NWAVES; ++j) {
-      const int idx = wave + j * C::NWAVES;
-      copy_b128_to_lds(rb, base + C::A_BYTES + idx * 1024, b_voff + idx * OpB::RPI * (int)ld + dead);
-    }
-    if (EPI == EPI_BLOCK) {
-      // activation scales of this slab's rows: wave w fetches rows 64 w .. 64 w + 63 (spare waves issue
-      // an out-of-range copy so that every wave has the same number of copies in flight)
-      const i32x4_t rs = raw_rsrc(io.sa_base + (uint64_t)ktc * (uint64_t)p.m_total * 4, io.sa_bytes);
-      const int off = wave * 64 < C::BM ? (wave * 64 + lane) * 4 + dead : kNoFetch;
-      copy_b32_to_lds(rs, base + C::A_BYTES + C::B_BYTES + (wave * 64 < C::BM ? wave * 256 : C::BM * 4), off);
+  auto copy_k = [&](const SlabCopy& sc, int k) {
+    if (k < CS) {
+      // activation scales of the slab's rows: wave w fetches rows 64 w .. 64 w + 63; spare waves issue an
+      // out-of-range copy into a sink so that every wave has the same number of copies in flight
+      const bool mine = wave * 64 < C::BM;
+      copy_b32_to_lds(sc.rs, sc.base + C::A_BYTES + C::B_BYTES + (mine ? wave * 256 : C::BM * 4),
+                      mine ? (wave * 64 + lane) * 4 : kNoFetch);
+    } else if (k < CS + CA) {
+      const int idx = wave + (k - CS) * C::NWAVES;  // wave-uniform
+      copy_b128_to_lds(sc.ra, sc.base + idx * 1024, a_voff + idx * OpA::RPI * (int)ld);
+    } else {
+      const int idx = wave + (k - CS - CA) * C::NWAVES;
+      copy_b128_to_lds(sc.rb, sc.base + C::A_BYTES + idx * 1024, b_voff + idx * OpB::RPI * (int)ld);
     }
   };
 
-  char* const stage_c = smem + (C::NSTAGE - 1) * C::STAGE_BYTES + wave * C::EPI_WAVE_BYTES;
+  char* const stage_c = smem + C::EPI_OFF + wave * C::EPI_WAVE_BYTES;
 
-  const TileWalk walk = sched_walk(num_tiles, !KGROUP && p.tile_split);
-  int64_t tile_id = walk.first;
-  Tile t;
-  TileIo io;
-  float sbv = 0.f;
-  if (tile_id < walk.end) {
-    t = sched_tile<C::BM, C::BN>(p, sched, tile_id);
-    io = make_io(t);
-    sbv = load_sbv(t);
-    asm volatile("" : "+v"(sbv));
+  // Software pipeline.  A slab is worked off in TM x 2 cells (32-row block i, 32-column block j), two
+  // 64-deep multiplies each.  The B fragments of both column blocks stay in registers for the slab, the
+  // A fragments of row block i+1 are read during row block i.  Before the last cell (TM-1, 1): wait for
+  // this wave's share of the next slab, workgroup barrier, read the next slab's j = 0 and i = 0
+  // fragments (the registers of the current slab's j = 0 fragments are free by then), then multiply;
+  // the next slab's j = 1 fragments follow during its first cell.  The copies of the slab after the
+  // next one are issued one per multiply from that point on (see gemm_fast.hip for why).
+  feed_seek(walk.first);
+  {
+    const SlabCopy s0 = begin_slab(0);
 #pragma unroll
-    for (int s = 0; s < C::NSTAGE - 1; ++s) issue_slab(io, s, s);
+    for (int k = 0; k < NC; ++k) copy_k(s0, k);
   }
-  while (tile_id < walk.end) {
-    const int64_t next_id = tile_id + walk.stride;
-    Tile nt = t;
-    float sbv_next = 0.f;
-    if (next_id < walk.end) {
-      nt = sched_tile<C::BM, C::BN>(p, sched, next_id);
+  wait_vmcnt<0>();
+  __syncthreads();
+  SlabCopy sc = begin_slab(1);
+  // copy k of `sc`, if there is one (k is a compile-time constant at every call site)
+  auto copy_at = [&](int k) {
+    if (k < NC) {
+      __builtin_amdgcn_sched_barrier(0);
+      copy_k(sc, k);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  copy_at(0);
+  copy_at(1);
+  i32x8_t fb0[2], fb1[2], fax[2], fay[2];
+  load_frag(smem + C::A_BYTES + wn0 * 128, fb0);
+  load_frag(smem + wm0 * 128, fax);
+  int ring = 0;
+
+  Tile nt;
+  float sbv_next = 0.f;
+  if (walk.first < walk.end) {
+    nt = sched_tile<C::BM, C::BN>(p, sched, walk.first);
+    sbv_next = load_sbv(nt);
+  }
+  for (int64_t tile_id = walk.first; tile_id < walk.end; tile_id += walk.stride) {
+    const Tile cur = nt;
+    const int kt_n = __builtin_amdgcn_readfirstlane(slabs_of(cur));
+    float sbv = sbv_next;
+    if (tile_id + walk.stride < walk.end) {
+      nt = sched_tile<C::BM, C::BN>(p, sched, tile_id + walk.stride);
       sbv_next = load_sbv(nt);
     }
     f32x16_t acc[C::TM][C::TN];
@@ -176,71 +240,76 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    const int kt_n = io.kt_n;
     for (int kt = 0; kt < kt_n; ++kt) {
-      wait_vmcnt<LPW * (C::NSTAGE - 2)>();
-      __syncthreads();
-      issue_slab(io, kt + C::NSTAGE - 1, (kt + C::NSTAGE - 1) % C::NSTAGE);
-      const float sb_cur = EPI == EPI_BLOCK ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sbv), kt)) : 1.f;
-      const char* sa = smem + (kt % C::NSTAGE) * C::STAGE_BYTES + wm0 * 128;
-      const char* sb = smem + (kt % C::NSTAGE) * C::STAGE_BYTES + C::A_BYTES + wn0 * 128;
-      const float* ss = (const float*)(smem + (kt % C::NSTAGE) * C::STAGE_BYTES + C::A_BYTES + C::B_BYTES) + wm0 + l32;
-
-      i32x8_t fb[2][C::TN];
+      const char* sa = smem + (ring & 1) * C::STAGE_BYTES;
+      const char* sn = smem + ((ring + 1) & 1) * C::STAGE_BYTES;
+      float srow[C::TM];
+      if (BLOCK) {
+        const float sb_cur = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sbv), kt));
+        const float* ss = (const float*)(sa + C::A_BYTES + C::B_BYTES) + wm0 + l32;
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks)
+        for (int i = 0; i < C::TM; ++i) srow[i] = ss[32 * i] * sb_cur;
+      }
+      // one cell: two multiplies, with `mid` run right after the first has been issued; copies k0 and
+      // k0 + 1 of the slab being requested go out after the first and the second multiply
+      auto cell = [&](int i, int j, int k0, const i32x8_t (&fa)[2], const i32x8_t (&fb)[2], auto&& mid) {
+        if (BLOCK) {
+          f32x16_t part = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+          part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[0], fa[0], part, FB, FA, 0, 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          mid();
+          copy_at(k0);
+          __builtin_amdgcn_sched_barrier(0);
+          part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[1], fa[1], part, FB, FA, 0, 0, 0, 0);
+          copy_at(k0 + 1);
+          // the empty asm statements pin the scaling between the multiplies of this cell and the next one
+          // (plain arithmetic is otherwise free to drift, which keeps many partial tiles alive at once)
+          asm volatile("" : "+v"(part));
 #pragma unroll
-        for (int j = 0; j < C::TN; ++j) {
-          const i32x4_t lo = *(const i32x4_t*)(sb + rd[ks][0] + j * 32 * 128);
-          const i32x4_t hi = *(const i32x4_t*)(sb + rd[ks][1] + j * 32 * 128);
-          fb[ks][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          for (int e = 0; e < 16; ++e) acc[i][j][e] += part[e] * srow[i];
+          asm volatile("" : "+v"(acc[i][j]));
+        } else {
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[0], fa[0], acc[i][j], FB, FA, 0, 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+          mid();
+          copy_at(k0);
+          __builtin_amdgcn_sched_barrier(0);
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[1], fa[1], acc[i][j], FB, FA, 0, 0, 0, 0);
+          copy_at(k0 + 1);
         }
+        __builtin_amdgcn_sched_barrier(0);
+      };
 #pragma unroll
-      for (int i = 0; i < C::TM; ++i) {
-        i32x8_t fa[2];
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-          const i32x4_t lo = *(const i32x4_t*)(sa + rd[ks][0] + i * 32 * 128);
-          const i32x4_t hi = *(const i32x4_t*)(sa + rd[ks][1] + i * 32 * 128);
-          fa[ks] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
-        float s = 0.f;
-        if (EPI == EPI_BLOCK) s = ss[32 * i] * sb_cur;
-#pragma unroll
-        for (int j = 0; j < C::TN; ++j) {
-          if (EPI == EPI_BLOCK) {
-            f32x16_t part = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-            part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[0][j], fa[0], part, FB, FA, 0, 0, 0, 0);
-            part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[1][j], fa[1], part, FB, FA, 0, 0, 0, 0);
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] += part[e] * s;
-          } else {
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[0][j], fa[0], acc[i][j], FB, FA, 0, 0, 0, 0);
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[1][j], fa[1], acc[i][j], FB, FA, 0, 0, 0, 0);
-          }
+      for (int i = 0; i < C::TM; i += 2) {
+        // row block i from fax, i + 1 from fay; cell c of the slab issues copies 2 + 2 c and 3 + 2 c
+        cell(i, 0, 2 + 4 * i, fax, fb0, [&] {
+          if (i == 0) load_frag(sa + C::A_BYTES + (wn0 + 32) * 128, fb1);
+          load_frag(sa + (wm0 + 32 * (i + 1)) * 128, fay);
+        });
+        cell(i, 1, 4 + 4 * i, fax, fb1, [&] {});
+        if (i + 2 < C::TM) {
+          cell(i + 1, 0, 6 + 4 * i, fay, fb0, [&] { load_frag(sa + (wm0 + 32 * (i + 2)) * 128, fax); });
+          cell(i + 1, 1, 8 + 4 * i, fay, fb1, [&] {});
+        } else {
+          cell(i + 1, 0, 6 + 4 * i, fay, fb0, [&] {});
+          const SlabCopy scn = begin_slab(ring & 1);  // scalar work only: overlaps the multiplies in flight
+          wait_vmcnt<0>();
+          if (BLOCK) asm volatile("" : "+v"(sbv_next));  // nothing of this wave is in flight: touching it costs no wait
+          __syncthreads();
+          sc = scn;
+          load_frag(sn + C::A_BYTES + wn0 * 128, fb0);
+          load_frag(sn + wm0 * 128, fax);
+          __builtin_amdgcn_sched_barrier(0);
+          cell(i + 1, 1, 0, fay, fb1, [&] {});
         }
       }
+      ++ring;
     }
-    wait_vmcnt<0>();
-    asm volatile("" : "+v"(sbv_next));
-    sbv = sbv_next;
-    __syncthreads();
-
-    const Tile cur = t;
-    if (next_id < walk.end) {
-      t = nt;
-      io = make_io(t);
-#pragma unroll
-      for (int s = 0; s < C::NSTAGE - 1; ++s) issue_slab(io, s, s);
-    }
-    tile_id = next_id;
 
     // Epilogue (see gemm_fast.hip): per-channel scaling happens on the fp32 values before packing.
-    constexpr int WCOLS = C::BN / C::WN, CPRW = WCOLS / 8, RPIW = 64 / CPRW;
     const int64_t c_row0 = KGROUP ? ((int64_t)cur.g * p.m_total + cur.row0) : cur.row0;
     char* const c_tile = (char*)p.C + ((c_row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2;
-    const int st_row = lane / CPRW, st_chunk = lane % CPRW;
-    const bool col_ok = cur.n0 + wn0 + st_chunk * 8 < p.N;
+    const int st_row = lane >> 2, st_chunk = lane & 3;
 #pragma unroll
     for (int i = 0; i < C::TM; ++i) {
       float rs = 1.f;
@@ -249,7 +318,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
         rs = m < cur.rows ? p.scale_m[(KGROUP ? (int64_t)cur.g * p.scale_m_sg : 0) + cur.row0 + m] : 0.f;
       }
 #pragma unroll
-      for (int j = 0; j < C::TN; ++j)
+      for (int j = 0; j < C::TN; ++j) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           float v[4];
@@ -260,17 +329,20 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] = (n + e < p.N) ? v[e] * rs * p.scale_n[(int64_t)cur.g * p.N + n + e] : 0.f;
           }
-          *(uint2*)(stage_c + l32 * C::EPI_PITCH + (32 * j + 8 * q + 4 * lh) * 2) = pack4<OUT>(v[0], v[1], v[2], v[3]);
+          *(uint2*)(stage_c + l32 * C::EPI_PITCH + (8 * q + 4 * lh) * 2) = pack4<OUT>(v[0], v[1], v[2], v[3]);
         }
+        const bool col_ok = cur.n0 + wn0 + 32 * j + st_chunk * 8 < p.N;
 #pragma unroll
-      for (int it = 0; it < 32 / RPIW; ++it) {
-        const int r = it * RPIW + st_row;
-        const i32x4_t v = *(const i32x4_t*)(stage_c + r * C::EPI_PITCH + st_chunk * 16);
-        if (col_ok && wm0 + 32 * i + r < cur.rows)
-          *(i32x4_t*)(c_tile + ((int64_t)(32 * i + r) * p.N + st_chunk * 8) * 2) = v;
+        for (int it = 0; it < 2; ++it) {
+          const int r = it * 16 + st_row;
+          const i32x4_t v = *(const i32x4_t*)(stage_c + r * C::EPI_PITCH + st_chunk * 16);
+          if (col_ok && wm0 + 32 * i + r < cur.rows)
+            *(i32x4_t*)(c_tile + ((int64_t)(32 * i + r) * p.N + 32 * j + st_chunk * 8) * 2) = v;
+        }
       }
     }
   }
+  wait_vmcnt<0>();  // the trailing zero-length copies still write LDS: let them finish before the wave ends
 }
 
 template <class C, int FA, int FB, int EPI, int OUT, bool KGROUP>
@@ -290,7 +362,7 @@ int launch_fp8_cfg(const GemmParams& p, hipStream_t s) {
   return check_launch("gemm_fp8");
 }
 
-typedef Fp8Cfg<256, 256, 2, 2, 4> Fp8Default;
+typedef Fp8Cfg<256, 256, 2, 4> Fp8Default;
 
 template <int FA, int FB, bool KGROUP>
 int launch_channel_out(const GemmParams& p, int out_dt, hipStream_t s) {
