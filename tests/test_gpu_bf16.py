@@ -49,6 +49,7 @@ def test_config1_tiny_reference_case(dev, variant):
     ([1, 0, 127, 129, 256, 3, 0, 300], 136, 72),
     ([0, 0, 5], 8, 8),
     ([200] * 16, 264, 64),
+    ([300, 0, 417], 2600, 128),  # 11 (tuned) / 21 (generic) column tiles: the tile order's last chunk is narrower
 ])
 def test_m_grouped_exact_on_integer_inputs(dev, variant, dtype, trans_b, sizes, N, K):
     """Entries in {-1,0,1}: every partial sum is an integer <= K <= 256, exactly representable, so the
@@ -163,6 +164,7 @@ def test_masked_full_mask_reduces_to_bmm_exact(dev, variant):
     ([128, 256, 0, 64], 256, 128),
     ([1, 33, 0, 130, 7], 136, 72),
     ([512], 128, 384),
+    ([40, 0, 200], 520, 2600),  # ragged last chunk of the tile order, three row tiles
 ])
 def test_k_grouped_exact_on_integer_inputs(dev, variant, dtype, sizes, Mdim, N):
     """Entries in {-1,0,1} and every group <= 512 tokens... sums stay below 256 in magnitude with

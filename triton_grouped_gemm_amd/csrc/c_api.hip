@@ -13,6 +13,7 @@ static thread_local char g_err[512] = "";
 static int g_force_generic = 0;
 static int g_tile_split = 1;
 static int g_store_nt = 0;
+static int g_n_chunk = 0;
 
 int set_error(const char* fmt, ...) {
   va_list ap;
@@ -65,6 +66,7 @@ static GemmParams zero_params() {
   memset(&p, 0, sizeof(p));
   p.tile_split = g_tile_split;
   p.store_nt = g_store_nt;
+  p.n_chunk = g_n_chunk;
   return p;
 }
 
@@ -245,6 +247,7 @@ int tgg_set_option(const char* key, int value) {
   if (key && strcmp(key, "force_generic") == 0) { g_force_generic = value != 0; return 0; }
   if (key && strcmp(key, "variant") == 0) { set_fast_variant(value); return 0; }
   if (key && strcmp(key, "tile_split") == 0) { g_tile_split = value != 0; return 0; }
+  if (key && strcmp(key, "n_chunk") == 0) { g_n_chunk = value < 0 ? 0 : value; return 0; }
   if (key && strcmp(key, "store_nt") == 0) { g_store_nt = value != 0; return 0; }
   return set_error("unknown option '%s'", key ? key : "(null)");
 }

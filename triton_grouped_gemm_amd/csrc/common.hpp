@@ -85,6 +85,7 @@ struct GemmParams {
   int K;                  // reduction length (M-grouped); unused for K-grouped
   int grid_limit;         // >0 caps the persistent grid
   int tile_split;         // tuned kernels: 1 = per-XCD contiguous tile ranges (see sched_walk)
+  int n_chunk;            // column tiles per chunk of the tile order, 0 = automatic (see sched_tile)
   int store_nt;           // tuned kernels: 1 = non-temporal output stores
 };
 

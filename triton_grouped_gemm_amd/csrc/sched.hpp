@@ -87,18 +87,47 @@ TGG_DEV int64_t sched_num_tiles(const GemmParams& p, const Table& t) {
   return (int64_t)t.tile0[p.G] * tiles_n;
 }
 
+// Tile order.  Consecutive tile ids are handed to workgroups that run at the same time on one XCD
+// (see sched_walk), so a run of ids should cover a near-square block of tiles: a run of R tiles spanning
+// w column tiles touches R / w row panels of A plus w column panels of B per K slab.  The N tiles are
+// therefore cut into chunks of at most eight columns and ids run over (chunk, row tile, column within
+// chunk), innermost last.  Eight rather than the square root of an XCD's 32 workgroups: B panels
+// (weights) are reused by the following row tiles of the group, A panels are streamed once, so the
+// wider side goes to B.
+TGG_DEV int sched_chunk_width(int tiles_n, int n_chunk) {
+  if (n_chunk > 0) return n_chunk < tiles_n ? n_chunk : tiles_n;
+  const int chunks = (tiles_n + 7) / 8;
+  return (tiles_n + chunks - 1) / chunks;
+}
+
+// Splits the position `r` inside a block of `rows_m` row tiles x `tiles_n` column tiles into (row tile, column tile).
+TGG_DEV void sched_split(int r, int rows_m, int tiles_n, int nc, int& mt, int& nt) {
+  const int chunk_tiles = rows_m * nc;
+  int c = r / chunk_tiles;
+  const int full = tiles_n / nc;
+  int width = nc;
+  if (c >= full) {  // the last, narrower chunk
+    c = full;
+    width = tiles_n - full * nc;
+  }
+  const int q = r - c * chunk_tiles;
+  mt = q / width;
+  nt = c * nc + (q - mt * width);
+}
+
 template <int BM, int BN, class Table>
 TGG_DEV Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id) {
   Tile r;
   const int tiles_n = (p.N + BN - 1) / BN;
+  const int nc = sched_chunk_width(tiles_n, p.n_chunk);
+  const int tid32 = (int)tile_id;  // the tile space is far below 2^31; 32-bit division is much cheaper
   if (p.mode == MODE_KG || p.mode == MODE_KG_COUNT) {
     const int tiles_m = (int)((p.m_total + BM - 1) / BM);
     const int per_group = tiles_m * tiles_n;
-    const int tid32 = (int)tile_id;
     r.g = tid32 / per_group;
-    const int rem = tid32 % per_group;
-    const int mt = rem / tiles_n;
-    r.n0 = (rem % tiles_n) * BN;
+    int mt, nt;
+    sched_split(tid32 - r.g * per_group, tiles_m, tiles_n, nc, mt, nt);
+    r.n0 = nt * BN;
     r.row0 = (int64_t)mt * BM;
     const int64_t left = p.m_total - r.row0;
     r.rows = left < BM ? (int)left : BM;
@@ -106,9 +135,9 @@ TGG_DEV Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id) {
     r.k1 = r.k0 + t.rows[r.g];
     return r;
   }
-  const int tid32 = (int)tile_id;  // the tile space is far below 2^31; 32-bit division is much cheaper
-  const int mt_glob = tid32 / tiles_n;
-  r.n0 = (tid32 % tiles_n) * BN;
+  int mt_glob, nt;
+  sched_split(tid32, t.tile0[p.G], tiles_n, nc, mt_glob, nt);
+  r.n0 = nt * BN;
   int lo = 0, hi = p.G;  // last g with tile0[g] <= mt_glob
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
