@@ -24,6 +24,21 @@ sys.path.insert(0, ROOT)
 PEAK_TFLOPS = {"bf16": 2500.0, "fp8": 5000.0}   # MI355X dense MFMA peaks
 PEAK_HBM_GBS = 8000.0
 
+# HBM-side bytes per launch of each workload's kernel in GB, measured offline with rocprofv3
+# (--pmc FETCH_SIZE and --pmc WRITE_SIZE, one counter per run, each scaled by what the counter reads for a
+# plain 1 GiB device copy: x2.0 and x1.0).  The runs and their figures are listed in profiles/hbm_traffic.txt.
+# FETCH_SIZE includes L2 fills served by the memory-side cache, so these are upper bounds on DRAM traffic.
+MEASURED_TRAFFIC_GB = {
+    "bf16_m_grouped_gateup_nt": 12.65,
+    "bf16_m_grouped_gateup_nn": 12.00,
+    "bf16_m_grouped_down_nt": 6.27,
+    "bf16_m_grouped_down_nn": 6.18,
+    "bf16_masked_decode": 2.59,
+    "bf16_k_grouped_wgrad": 40.54,
+    "fp8_block_m_grouped": 21.50,
+    "quant_trans128": 8.12,
+}
+
 G, M_TOTAL = 128, 655360
 WORKLOADS = {
     # name: (kind, N, K, trans_b)
@@ -38,7 +53,7 @@ WORKLOADS = {
 }
 
 
-def build_workload(name: str, dev, seed: int = 2026):
+def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu: int = -1):
     """Returns (fn, flops_per_step, algorithmic_bytes_per_step, dtype_tag, description, cpu_sample_fn)."""
     from triton_grouped_gemm_amd import workloads as wl
     from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm_TMA import m_grouped_gemm
@@ -48,7 +63,10 @@ def build_workload(name: str, dev, seed: int = 2026):
     if kind == "mg":
         a = wl.randn_bf16((M_TOTAL, K), K ** -0.5, seed + 1, dev)
         b = wl.randn_bf16((G, N, K) if trans_b else (G, K, N), K ** -0.5, seed + 2, dev)
-        fn = lambda: m_grouped_gemm(a, b, sizes, trans_b)
+        if zeros:  # same kernel, same traffic, no switching activity in the multipliers
+            a.zero_()
+            b.zero_()
+        fn = lambda: m_grouped_gemm(a, b, sizes, trans_b, numSM=num_cu)
         flops = 2.0 * M_TOTAL * N * K
         nbytes = 2.0 * M_TOTAL * K + 2.0 * G * N * K + 2.0 * M_TOTAL * N
 
@@ -129,6 +147,11 @@ def main() -> int:
     ap.add_argument("--workload", default="bf16_m_grouped_gateup_nt", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="host-core time budget of the CPU baseline sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--zeros", action="store_true",
+                    help="M-grouped bf16 workloads only: all-zero operands (diagnostic: shows how far the clock is held down "
+                         "by the power the multipliers draw on random data); reported as data=synthetic-zeros")
+    ap.add_argument("--num-cu", type=int, default=-1,
+                    help="M-grouped bf16 workloads only: cap the persistent grid at this many workgroups (diagnostic)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy (reference kernel for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -142,7 +165,12 @@ def main() -> int:
     _native.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    fn, flops, nbytes, dtype_tag, config, cpu_sample = build_workload(args.workload, dev)
+    if (args.zeros or args.num_cu > 0) and WORKLOADS[args.workload][0] != "mg":
+        print("--zeros / --num-cu apply to the bf16_m_grouped_* workloads only", file=sys.stderr)
+        return 2
+    fn, flops, nbytes, dtype_tag, config, cpu_sample = build_workload(args.workload, dev, zeros=args.zeros, num_cu=args.num_cu)
+    if args.num_cu > 0:
+        config["num_cu"] = args.num_cu
 
     if args.copy_calibration:
         src = torch.empty(1 << 28, device=dev, dtype=torch.float32).normal_()
@@ -166,12 +194,14 @@ def main() -> int:
     avg_kernel_ms = sum(kernel_ms) / len(kernel_ms)
 
     is_gemm = flops > 0
+    traffic = MEASURED_TRAFFIC_GB.get(args.workload)
+    traffic = None if traffic is None else round(traffic * 1e9)  # bytes per launch
     if is_gemm:
         value = flops / (wall_ms * 1e-3) / 1e12
         peak = PEAK_TFLOPS["fp8" if dtype_tag == "fp8" else "bf16"]
         achieved = flops / (avg_kernel_ms * 1e-3) / 1e12
         roofline = dict(bound="mfma", achieved=round(achieved, 2), peak=peak, unit="TFLOP/s",
-                        frac=round(achieved / peak, 4), traffic=None,
+                        frac=round(achieved / peak, 4), traffic=traffic,
                         min_ms=round(min(kernel_ms), 4), avg_ms=round(avg_kernel_ms, 4),
                         algorithmic_gbytes=round(nbytes / 1e9, 3))
         metric, unit = "grouped GEMM TFLOP/s (2*M*N*K/time), M-grouped G=128", "TFLOP/s"
@@ -179,7 +209,7 @@ def main() -> int:
         value = nbytes / (wall_ms * 1e-3) / 1e9
         achieved = nbytes / (avg_kernel_ms * 1e-3) / 1e9
         roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit="GB/s",
-                        frac=round(achieved / PEAK_HBM_GBS, 4), traffic=None,
+                        frac=round(achieved / PEAK_HBM_GBS, 4), traffic=traffic,
                         min_ms=round(min(kernel_ms), 4), avg_ms=round(avg_kernel_ms, 4))
         metric, unit = "quantizer algorithmic GB/s", "GB/s"
 
@@ -192,7 +222,7 @@ def main() -> int:
     print(json.dumps({
         "metric": metric, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": dtype_tag, "data": "synthetic", "config": config,
+        "vs_baseline": None, "dtype": dtype_tag, "data": "synthetic-zeros" if args.zeros else "synthetic", "config": config,
         "roofline": roofline, "cpu_baseline": cpu_baseline,
     }))
     return 0
