@@ -97,8 +97,12 @@ int tgg_per_block_cast_to_fp8(const void* x, void* codes, float* scales, int bat
  * `.to(torch.float8_*)` casts of the recipes above). */
 int tgg_cvt_f32_to_fp8(const float* in, void* out, int64_t n, int fmt, void* stream);
 
-/* Library controls: "force_generic" (0/1) routes every GEMM through the shape-agnostic kernel;
- * "variant" (int) selects a tile configuration of the tuned 16-bit kernels (0 = default). */
+/* Library controls (process-wide, meant for tests and tuning; returns 1 for an unknown key):
+ *   "force_generic" 0/1  route every GEMM through the shape-agnostic kernel
+ *   "variant"       int  tile configuration of the tuned 16-bit kernels (0 = 256x256 default, 1 = 256x128)
+ *   "tile_split"    0/1  16-bit M-grouped: per-XCD contiguous tile ranges (default 1) or interleaved sweeps
+ *   "n_chunk"       int  column tiles per chunk of the tile order (0 = automatic, at most eight)
+ *   "store_nt"      0/1  write the output with non-temporal stores (default 0) */
 int tgg_set_option(const char* key, int value);
 const char* tgg_last_error(void);
 int tgg_version(void);
