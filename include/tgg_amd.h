@@ -97,6 +97,17 @@ int tgg_per_block_cast_to_fp8(const void* x, void* codes, float* scales, int bat
  * `.to(torch.float8_*)` casts of the recipes above). */
 int tgg_cvt_f32_to_fp8(const float* in, void* out, int64_t n, int fmt, void* stream);
 
+/* Test hook, runs entirely on the host (no GPU needed): the order in which `grid` persistent workgroups walk
+ * the output tiles of a launch, computed by the same scheduler functions the kernels execute.  It restates
+ * what the reference's grouped_launch / m_indices_pad tile enumeration guarantees
+ * (gemm/BF16/m_grouped_gemm_TMA.py:55-71, :297-326): every tile of the padded tile space exactly once.
+ *   sizes  host array [G]; mode 0 M-grouped, 1 rows padded to `aux`, 2 masked with `aux` rows per group,
+ *          4 K-grouped by token counts (`aux` = total tokens, m_total = rows of each output)
+ *   tile   256 (tuned kernels) or 128 (shape-agnostic kernel); split as in the "tile_split" option
+ *   out    [capacity][6] = workgroup, position in its walk, group, first row, valid rows, first column */
+int tgg_debug_tile_order(const int64_t* sizes, int G, int mode, int64_t m_total, int64_t aux, int N, int tile,
+                         int grid, int split, int64_t* out, int64_t capacity, int64_t* num_tiles);
+
 /* Library controls (process-wide, meant for tests and tuning; returns 1 for an unknown key):
  *   "force_generic" 0/1  route every GEMM through the shape-agnostic kernel
  *   "variant"       int  tile configuration of the tuned 16-bit kernels (0 = 256x256 default, 1 = 256x128)

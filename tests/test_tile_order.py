@@ -1,0 +1,108 @@
+"""The persistent kernels' tile scheduler, run on the host through the library's test hook (no GPU):
+every output tile of the grouped tile space is visited exactly once, whatever the group sizes, grid size,
+walk and chunking.  This is the invariant the reference's tile enumeration provides
+(gemm/BF16/m_grouped_gemm_TMA.py:55-71 grouped_launch, :297-326 m_indices_pad); results do not depend on
+the order, only on the cover."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from triton_grouped_gemm_amd import _native
+
+MG, MG_PAD, MASKED, KG_COUNT = 0, 1, 2, 4
+
+
+def tile_order(sizes, mode, m_total, aux, N, tile, grid, split, n_chunk=0):
+    lib = _native.load()
+    _native.set_option("n_chunk", n_chunk)
+    try:
+        s = np.asarray(sizes, dtype=np.int64)
+        cap = 1 << 16
+        out = np.zeros((cap, 6), dtype=np.int64)
+        n = ctypes.c_int64(0)
+        rc = lib.tgg_debug_tile_order(s.ctypes.data, len(s), mode, m_total, aux, N, tile, grid, split,
+                                      out.ctypes.data, cap, ctypes.byref(n))
+        assert rc == 0, lib.tgg_last_error().decode()
+        return out[:n.value], n.value
+    finally:
+        _native.set_option("n_chunk", 0)
+
+
+def expected_m_grouped_tiles(sizes, starts, tile, N, m_total):
+    exp = set()
+    for g, (sz, st) in enumerate(zip(sizes, starts)):
+        sz = max(0, min(sz, m_total - st))
+        for mt in range(-(-sz // tile)):
+            rows = min(tile, sz - mt * tile)
+            for nt in range(-(-N // tile)):
+                exp.add((g, st + mt * tile, rows, nt * tile))
+    return exp
+
+
+@pytest.mark.parametrize("tile", [256, 128])
+@pytest.mark.parametrize("split", [0, 1])
+@pytest.mark.parametrize("grid", [256, 64, 7, 1])
+@pytest.mark.parametrize("n_chunk", [0, 1, 3])
+@pytest.mark.parametrize("sizes,N", [
+    ([64, 128, 32, 96], 512),
+    ([1, 0, 127, 129, 256, 3, 0, 300], 136),
+    ([300, 0, 417], 2600),
+    ([5120] * 16, 1536),
+    ([0, 0, 0], 256),
+])
+def test_m_grouped_cover(tile, split, grid, n_chunk, sizes, N):
+    starts = np.concatenate([[0], np.cumsum(sizes)[:-1]]).tolist()
+    rows, n = tile_order(sizes, MG, sum(sizes), 0, N, tile, grid, split, n_chunk)
+    exp = expected_m_grouped_tiles(sizes, starts, tile, N, sum(sizes))
+    got = [tuple(r[2:6]) for r in rows.tolist()]
+    assert n == len(exp) == len(got)
+    assert set(got) == exp and len(set(got)) == len(got)
+    # positions inside a workgroup's walk are 0, 1, 2, ... and workgroup ids stay below the grid
+    for b in range(grid):
+        pos = rows[rows[:, 0] == b][:, 1]
+        assert pos.tolist() == list(range(len(pos)))
+    assert rows[:, 0].max(initial=0) < grid
+
+
+def test_padded_and_masked_starts():
+    sizes = [100, 0, 130, 128]
+    rows, n = tile_order(sizes, MG_PAD, 128 + 0 + 256 + 128, 128, 256, 256, 256, 1)
+    exp = expected_m_grouped_tiles(sizes, [0, 128, 128, 384], 256, 256, 512)
+    assert {tuple(r[2:6]) for r in rows.tolist()} == exp and n == len(exp)
+    masked = [512, 0, 77, 300]
+    rows, n = tile_order(masked, MASKED, 4 * 512, 512, 4096, 256, 256, 1)
+    exp = expected_m_grouped_tiles(masked, [0, 512, 1024, 1536], 256, 4096, 2048)
+    assert {tuple(r[2:6]) for r in rows.tolist()} == exp and n == len(exp)
+
+
+def test_rows_past_the_end_of_a_are_clipped():
+    """sizes that sum past m_total: the last group is cut, later ones vanish (never touch rows outside A)."""
+    rows, n = tile_order([200, 200, 200], MG, 300, 0, 256, 256, 256, 1)
+    assert {tuple(r[2:6]) for r in rows.tolist()} == {(0, 0, 200, 0), (1, 200, 100, 0)}
+
+
+@pytest.mark.parametrize("tile", [256, 128])
+@pytest.mark.parametrize("grid", [256, 24])
+def test_k_grouped_cover(tile, grid):
+    """K-grouped: every (group, row tile, column tile) of the [G, Mdim, N] output once, empty groups included
+    (their tiles must be written with zeros)."""
+    sizes, mdim, N = [40, 0, 200, 64], 520, 2600
+    rows, n = tile_order(sizes, KG_COUNT, mdim, sum(sizes), N, tile, grid, 0)
+    exp = {(g, mt * tile, min(tile, mdim - mt * tile), nt * tile)
+           for g in range(len(sizes)) for mt in range(-(-mdim // tile)) for nt in range(-(-N // tile))}
+    got = [tuple(r[2:6]) for r in rows.tolist()]
+    assert n == len(exp) and set(got) == exp and len(set(got)) == len(got)
+
+
+def test_runs_of_an_xcd_are_near_square():
+    """With 256 workgroups dealt round robin to 8 XCDs, the 32 tiles an XCD works on at the same time should
+    span few distinct row panels and column panels (this is what keeps operand re-reads inside one L2)."""
+    sizes, N = [5120] * 128, 4096  # 16 column tiles -> chunks of 8
+    rows, _ = tile_order(sizes, MG, sum(sizes), 0, N, 256, 256, 1)
+    first = rows[rows[:, 1] == 0]
+    for x in range(8):
+        mine = first[first[:, 0] % 8 == x]
+        assert len(mine) == 32
+        assert len(set(mine[:, 3].tolist())) * len(set(mine[:, 5].tolist())) == 32  # a full rectangle
+        assert len(set(mine[:, 3].tolist())) + len(set(mine[:, 5].tolist())) <= 12   # 4 x 8

@@ -6,6 +6,7 @@
 #include "../../include/tgg_amd.h"
 #include "common.hpp"
 #include "launch.hpp"
+#include "sched.hpp"
 
 namespace tgg {
 
@@ -78,6 +79,31 @@ static int dispatch_16bit(const GemmParams& p, int dt, int layout, hipStream_t s
 }  // namespace tgg
 
 using namespace tgg;
+
+// Host-side run of the device scheduler (same functions, see sched.hpp).
+template <int BM, int BN>
+static int tile_order_host(const GemmParams& p, int grid, int split, int64_t* out, int64_t capacity, int64_t* num_tiles) {
+  SchedTable* t = new SchedTable;
+  for (int g = 0; g < p.G; ++g) sched_load_group(p, *t, g);
+  sched_prefix<BM>(p, *t);
+  const int64_t total = sched_num_tiles<BM, BN>(p, *t);
+  *num_tiles = total;
+  int64_t n = 0;
+  for (int b = 0; b < grid; ++b) {
+    const TileWalk w = sched_walk_of(total, split != 0, grid, b);
+    int64_t pos = 0;
+    for (int64_t id = w.first; id < w.end; id += w.stride, ++pos) {
+      if (n < capacity) {
+        const Tile tl = sched_tile<BM, BN>(p, *t, id);
+        int64_t* r = out + n * 6;
+        r[0] = b; r[1] = pos; r[2] = tl.g; r[3] = tl.row0; r[4] = tl.rows; r[5] = tl.n0;
+      }
+      ++n;
+    }
+  }
+  delete t;
+  return n <= capacity ? 0 : set_error("tile order needs %lld rows, capacity %lld", (long long)n, (long long)capacity);
+}
 
 extern "C" {
 
@@ -241,6 +267,29 @@ int tgg_per_block_cast_to_fp8(const void* x, void* codes, float* scales, int bat
 int tgg_cvt_f32_to_fp8(const float* in, void* out, int64_t n, int fmt, void* stream) {
   if (!in || !out || n < 0) return set_error("bad arguments");
   return launch_cvt_fp8(in, out, n, fmt, (hipStream_t)stream);
+}
+
+int tgg_debug_tile_order(const int64_t* sizes, int G, int mode, int64_t m_total, int64_t aux, int N, int tile,
+                         int grid, int split, int64_t* out, int64_t capacity, int64_t* num_tiles) {
+  if (!sizes || !out || !num_tiles) return set_error("null pointer");
+  if (G < 1 || G > TGG_MAX_GROUPS) return set_error("G=%d outside [1, %d]", G, TGG_MAX_GROUPS);
+  if (N < 1 || grid < 1 || m_total < 0) return set_error("bad N / grid / m_total");
+  if (mode != MODE_MG && mode != MODE_MG_PAD && mode != MODE_MASKED && mode != MODE_KG_COUNT)
+    return set_error("mode %d not supported by the tile-order hook", mode);
+  GemmParams p = zero_params();
+  p.sizes = sizes;
+  p.sizes_i64 = 1;
+  p.G = G;
+  p.mode = mode;
+  p.m_total = m_total;
+  p.N = N;
+  p.align = mode == MODE_MG_PAD ? (int)aux : 1;
+  p.m_stride = mode == MODE_MASKED ? aux : 0;
+  p.k_total = mode == MODE_KG_COUNT ? aux : 0;
+  if (mode == MODE_MG_PAD && p.align < 1) return set_error("alignment must be positive");
+  if (tile == 256) return tile_order_host<256, 256>(p, grid, split, out, capacity, num_tiles);
+  if (tile == 128) return tile_order_host<128, 128>(p, grid, split, out, capacity, num_tiles);
+  return set_error("tile must be 256 (tuned kernels) or 128 (shape-agnostic kernel)");
 }
 
 int tgg_set_option(const char* key, int value) {

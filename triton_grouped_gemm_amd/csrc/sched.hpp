@@ -29,56 +29,68 @@ struct Tile {
   int64_t k1;
 };
 
-TGG_DEV int64_t load_size(const void* p, int is64, int i) {
+// The functions below that are marked TGG_HD contain no device-only construct: the library also runs them
+// on the host to report the tile order (a test hook), so what the tests check is what the kernels execute.
+#define TGG_HD __host__ __device__ __forceinline__
+
+TGG_HD int64_t load_size(const void* p, int is64, int i) {
   int64_t v = is64 ? ((const int64_t*)p)[i] : (int64_t)((const int32_t*)p)[i];
   return v < 0 ? 0 : v;
+}
+
+// Entry g of the table before the prefix pass: the group's raw extent.
+template <class Table>
+TGG_HD void sched_load_group(const GemmParams& p, Table& t, int g) {
+  if (p.mode == MODE_KG) {
+    int64_t s = p.k_start[g], e = p.k_end[g];
+    if (s < 0) s = 0;
+    if (e > p.k_total) e = p.k_total;
+    t.row0[g] = s;
+    t.rows[g] = e > s ? (int32_t)(e - s) : 0;
+  } else {
+    t.rows[g] = (int32_t)load_size(p.sizes, p.sizes_i64, g);
+  }
+}
+
+// Serial prefix pass over the loaded extents (every mode but MODE_KG, whose ranges are explicit).
+template <int BM, class Table>
+TGG_HD void sched_prefix(const GemmParams& p, Table& t) {
+  const int G = p.G;
+  int64_t row = 0;
+  int32_t tile = 0;
+  for (int g = 0; g < G; ++g) {
+    int64_t sz = t.rows[g];
+    int64_t start;
+    if (p.mode == MODE_MASKED) {
+      start = (int64_t)g * p.m_stride;
+      if (sz > p.m_stride) sz = p.m_stride;
+    } else {
+      start = row;
+      row += (p.mode == MODE_MG_PAD) ? ((sz + p.align - 1) / p.align) * p.align : sz;
+    }
+    const int64_t limit = (p.mode == MODE_KG_COUNT) ? p.k_total : p.m_total;
+    if (start >= limit) sz = 0;  // never touch rows (or k) past the end of the operands
+    else if (start + sz > limit) sz = limit - start;
+    t.row0[g] = start;
+    t.rows[g] = (int32_t)sz;
+    t.tile0[g] = tile;
+    tile += (int32_t)((sz + BM - 1) / BM);
+  }
+  t.tile0[G] = tile;
 }
 
 // All threads of the workgroup must call this; ends with a barrier.
 template <int BM, class Table>
 TGG_DEV void sched_init(const GemmParams& p, Table& t) {
-  const int G = p.G;
-  if (p.mode == MODE_KG) {
-    for (int g = threadIdx.x; g < G; g += blockDim.x) {
-      int64_t s = p.k_start[g], e = p.k_end[g];
-      if (s < 0) s = 0;
-      if (e > p.k_total) e = p.k_total;
-      t.row0[g] = s;
-      t.rows[g] = e > s ? (int32_t)(e - s) : 0;
-    }
-    __syncthreads();
-    return;
-  }
-  for (int g = threadIdx.x; g < G; g += blockDim.x) t.rows[g] = (int32_t)load_size(p.sizes, p.sizes_i64, g);
+  for (int g = threadIdx.x; g < p.G; g += blockDim.x) sched_load_group(p, t, g);
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int64_t row = 0;
-    int32_t tile = 0;
-    for (int g = 0; g < G; ++g) {
-      int64_t sz = t.rows[g];
-      int64_t start;
-      if (p.mode == MODE_MASKED) {
-        start = (int64_t)g * p.m_stride;
-        if (sz > p.m_stride) sz = p.m_stride;
-      } else {
-        start = row;
-        row += (p.mode == MODE_MG_PAD) ? ((sz + p.align - 1) / p.align) * p.align : sz;
-      }
-      const int64_t limit = (p.mode == MODE_KG_COUNT) ? p.k_total : p.m_total;
-      if (start >= limit) sz = 0;  // never touch rows (or k) past the end of the operands
-      else if (start + sz > limit) sz = limit - start;
-      t.row0[g] = start;
-      t.rows[g] = (int32_t)sz;
-      t.tile0[g] = tile;
-      tile += (int32_t)((sz + BM - 1) / BM);
-    }
-    t.tile0[G] = tile;
-  }
+  if (p.mode == MODE_KG) return;
+  if (threadIdx.x == 0) sched_prefix<BM>(p, t);
   __syncthreads();
 }
 
 template <int BM, int BN, class Table>
-TGG_DEV int64_t sched_num_tiles(const GemmParams& p, const Table& t) {
+TGG_HD int64_t sched_num_tiles(const GemmParams& p, const Table& t) {
   const int tiles_n = (p.N + BN - 1) / BN;
   if (p.mode == MODE_KG || p.mode == MODE_KG_COUNT) {
     const int tiles_m = (int)((p.m_total + BM - 1) / BM);
@@ -94,14 +106,14 @@ TGG_DEV int64_t sched_num_tiles(const GemmParams& p, const Table& t) {
 // chunk), innermost last.  Eight rather than the square root of an XCD's 32 workgroups: B panels
 // (weights) are reused by the following row tiles of the group, A panels are streamed once, so the
 // wider side goes to B.
-TGG_DEV int sched_chunk_width(int tiles_n, int n_chunk) {
+TGG_HD int sched_chunk_width(int tiles_n, int n_chunk) {
   if (n_chunk > 0) return n_chunk < tiles_n ? n_chunk : tiles_n;
   const int chunks = (tiles_n + 7) / 8;
   return (tiles_n + chunks - 1) / chunks;
 }
 
 // Splits the position `r` inside a block of `rows_m` row tiles x `tiles_n` column tiles into (row tile, column tile).
-TGG_DEV void sched_split(int r, int rows_m, int tiles_n, int nc, int& mt, int& nt) {
+TGG_HD void sched_split(int r, int rows_m, int tiles_n, int nc, int& mt, int& nt) {
   const int chunk_tiles = rows_m * nc;
   int c = r / chunk_tiles;
   const int full = tiles_n / nc;
@@ -116,7 +128,7 @@ TGG_DEV void sched_split(int r, int rows_m, int tiles_n, int nc, int& mt, int& n
 }
 
 template <int BM, int BN, class Table>
-TGG_DEV Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id) {
+TGG_HD Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id) {
   Tile r;
   const int tiles_n = (p.N + BN - 1) / BN;
   const int nc = sched_chunk_width(tiles_n, p.n_chunk);
@@ -166,8 +178,7 @@ struct TileWalk {
   int64_t first, end, stride;
 };
 
-TGG_DEV TileWalk sched_walk(int64_t num_tiles, bool split) {
-  const int P = gridDim.x, b = blockIdx.x;
+TGG_HD TileWalk sched_walk_of(int64_t num_tiles, bool split, int P, int b) {
   TileWalk w;
   if ((P & 7) != 0) {
     w.first = b; w.end = num_tiles; w.stride = P;
@@ -182,6 +193,10 @@ TGG_DEV TileWalk sched_walk(int64_t num_tiles, bool split) {
     w.stride = P;
   }
   return w;
+}
+
+TGG_DEV TileWalk sched_walk(int64_t num_tiles, bool split) {
+  return sched_walk_of(num_tiles, split, (int)gridDim.x, (int)blockIdx.x);
 }
 
 }  // namespace tgg
