@@ -66,6 +66,15 @@ template <int ROWS, bool KMAJOR> struct Operand {
     const int sw = KMAJOR ? (r / 2) % 8 : (r % 4) * 4;
     return r_local * ld + ((slot ^ sw) << 4);
   }
+  // K-contiguous rows only: which 16-byte chunk of its row (0..7) that lane fetches
+  static TGG_DEV int lane_chunk(int lane, int pat) {
+    const int r = pat * RPI + lane / CPR;
+    return (lane % CPR) ^ ((r / 2) % 8);
+  }
 };
+
+// A source offset no descriptor of the tuned kernels reaches (their operand windows stay below 1 GiB):
+// a lane given this offset fetches nothing and writes zeros.
+constexpr int kNoFetch = 0x40000000;
 
 }  // namespace tgg

@@ -99,6 +99,11 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   // per-lane source offsets of this wave's copies (one swizzle pattern per wave, see FastCfg)
   const int a_voff = OpA::lane_voff(lane, wave % OpA::NPAT, (int)a_ld);
   const int b_voff = OpB::lane_voff(lane, wave % OpB::NPAT, (int)b_ld);
+  // K tail (K not a multiple of the slab depth): in a tile's last slab the lanes whose 16-byte chunk of a
+  // K-contiguous row starts at or beyond K fetch nothing (zeros); token-row operands end with the descriptor.
+  const int tail_chunks = LAYOUT == LAYOUT_TN ? 0 : (p.K % BK) / 8;
+  const int a_voff_tail = (A_KMAJOR && OpA::lane_chunk(lane, wave % OpA::NPAT) >= tail_chunks) ? kNoFetch : a_voff;
+  const int b_voff_tail = (B_KMAJOR && OpB::lane_chunk(lane, wave % OpB::NPAT) >= tail_chunks) ? kNoFetch : b_voff;
 
   // per-lane LDS offsets of the fragment reads, relative to the operand's slab
   //   K-contiguous: 16 bytes = K values 16 ks + 8 lh + (0..7) of row (block + l32)
@@ -165,7 +170,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   const int64_t a_step = A_KMAJOR ? BK * 2 : BK * a_ld;
   const int64_t b_step = B_KMAJOR ? BK * 2 : BK * b_ld;
   auto slabs_of = [&](const Tile& t) -> int {
-    return LAYOUT == LAYOUT_TN ? (int)((t.k1 - t.k0 + BK - 1) / BK) : p.K / BK;
+    return LAYOUT == LAYOUT_TN ? (int)((t.k1 - t.k0 + BK - 1) / BK) : (p.K + BK - 1) / BK;
   };
   auto make_io = [&](const Tile& t) {
     TileIo io;
@@ -225,6 +230,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   struct SlabCopy {
     i32x4_t ra, rb;
     uint32_t base;
+    bool tail;  // the tile's last slab, cut short by K
   };
   constexpr int CA = C::NI_A / C::NWAVES, CB = C::NI_B / C::NWAVES, NC = CA + CB;
   constexpr int SP = (C::TM * C::TN) / (NC / 2);  // multiplies between two copies
@@ -235,6 +241,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
     sc.ra = make_rsrc(feed.a_base, live ? feed.a_left : 0);
     sc.rb = make_rsrc(feed.b_base, live ? feed.b_left : 0);
     sc.base = smem_addr + buf * C::STAGE_BYTES;
+    sc.tail = tail_chunks != 0 && feed.issued + 1 == feed.kt_n;
     feed.a_base += a_step;
     feed.a_left -= a_step;
     feed.b_base += b_step;
@@ -246,10 +253,10 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   auto copy_k = [&](const SlabCopy& sc, int k) {
     if (k < CA) {
       const int idx = wave + k * C::NWAVES;  // wave-uniform
-      copy_b128_to_lds(sc.ra, sc.base + idx * 1024, a_voff + idx * OpA::RPI * (int)a_ld);
+      copy_b128_to_lds(sc.ra, sc.base + idx * 1024, (sc.tail ? a_voff_tail : a_voff) + idx * OpA::RPI * (int)a_ld);
     } else {
       const int idx = wave + (k - CA) * C::NWAVES;
-      copy_b128_to_lds(sc.rb, sc.base + C::A_BYTES + idx * 1024, b_voff + idx * OpB::RPI * (int)b_ld);
+      copy_b128_to_lds(sc.rb, sc.base + C::A_BYTES + idx * 1024, (sc.tail ? b_voff_tail : b_voff) + idx * OpB::RPI * (int)b_ld);
     }
   };
 
@@ -407,7 +414,7 @@ bool fast_supported(const GemmParams& p, int dt, int layout) {
     return p.m_total * 2 * 64 < (1ll << 30) && (int64_t)p.N * 2 * 64 < (1ll << 30);
   }
   if (p.mode != MODE_MG && p.mode != MODE_MG_PAD && p.mode != MODE_MASKED) return false;
-  if (p.K < BK || (p.K % BK) != 0) return false;
+  if (p.K < 8 || (p.K & 7) != 0) return false;
   // per-lane source offsets stay far below the out-of-range marker
   if ((int64_t)p.K * 2 * 256 >= (1ll << 30)) return false;
   if (layout == LAYOUT_NN && (int64_t)p.N * 2 * 64 >= (1ll << 30)) return false;

@@ -72,6 +72,10 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
   const int64_t ld = KGROUP ? p.k_total : (int64_t)p.K;  // bytes between consecutive rows of A and of B
   const int a_voff = OpA::lane_voff(lane, wave % OpA::NPAT, (int)ld);
   const int b_voff = OpB::lane_voff(lane, wave % OpB::NPAT, (int)ld);
+  // K tail (see gemm_fast.hip): in a tile's last slab, chunks that start at or beyond K read as zero
+  const int tail_chunks = KGROUP ? 0 : (p.K % BKB) / 16;
+  const int a_voff_tail = OpA::lane_chunk(lane, wave % OpA::NPAT) >= tail_chunks ? kNoFetch : a_voff;
+  const int b_voff_tail = OpB::lane_chunk(lane, wave % OpB::NPAT) >= tail_chunks ? kNoFetch : b_voff;
   const int kblocks = (p.K + 127) >> 7;
   const int nblocks = (p.N + 127) >> 7;
 
@@ -99,7 +103,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
     int64_t a_left, b_left;
     int s_bytes, kt_n, issued;
   };
-  auto slabs_of = [&](const Tile& t) -> int { return KGROUP ? (int)((t.k1 - t.k0 + BKB - 1) / BKB) : p.K / BKB; };
+  auto slabs_of = [&](const Tile& t) -> int { return KGROUP ? (int)((t.k1 - t.k0 + BKB - 1) / BKB) : (p.K + BKB - 1) / BKB; };
   auto make_io = [&](const Tile& t) {
     TileIo io;
     const int64_t k0 = KGROUP ? t.k0 : 0;
@@ -150,6 +154,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
   struct SlabCopy {
     i32x4_t ra, rb, rs;
     uint32_t base;
+    bool tail;  // the tile's last slab, cut short by K
   };
   constexpr int CA = C::NI_A / C::NWAVES, CB = C::NI_B / C::NWAVES, CS = BLOCK ? 1 : 0, NC = CS + CA + CB;
   auto begin_slab = [&](int buf) {
@@ -159,6 +164,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
     sc.rb = make_rsrc(feed.b_base, live ? feed.b_left : 0);
     sc.rs = make_rsrc(feed.s_base, live ? feed.s_bytes : 0);
     sc.base = smem_addr + buf * C::STAGE_BYTES;
+    sc.tail = tail_chunks != 0 && feed.issued + 1 == feed.kt_n;
     feed.a_base += BKB;
     feed.a_left -= BKB;
     feed.b_base += BKB;
@@ -168,7 +174,6 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
     if (live && feed.issued >= feed.kt_n) feed_seek(feed_id + walk.stride);
     return sc;
   };
-  constexpr int kNoFetch = 0x40000000;
   auto copy_k = [&](const SlabCopy& sc, int k) {
     if (k < CS) {
       // activation scales of the slab's rows: wave w fetches rows 64 w .. 64 w + 63; spare waves issue an
@@ -178,10 +183,10 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
                       mine ? (wave * 64 + lane) * 4 : kNoFetch);
     } else if (k < CS + CA) {
       const int idx = wave + (k - CS) * C::NWAVES;  // wave-uniform
-      copy_b128_to_lds(sc.ra, sc.base + idx * 1024, a_voff + idx * OpA::RPI * (int)ld);
+      copy_b128_to_lds(sc.ra, sc.base + idx * 1024, (sc.tail ? a_voff_tail : a_voff) + idx * OpA::RPI * (int)ld);
     } else {
       const int idx = wave + (k - CS - CA) * C::NWAVES;
-      copy_b128_to_lds(sc.rb, sc.base + C::A_BYTES + idx * 1024, b_voff + idx * OpB::RPI * (int)ld);
+      copy_b128_to_lds(sc.rb, sc.base + C::A_BYTES + idx * 1024, (sc.tail ? b_voff_tail : b_voff) + idx * OpB::RPI * (int)ld);
     }
   };
 
@@ -392,7 +397,8 @@ bool fast_fp8_supported(const GemmParams& p, bool block_scaled) {
     return (p.k_total % BKB) == 0 && p.k_total * 256 < (1ll << 30);
   }
   if (p.mode != MODE_MG && p.mode != MODE_MG_PAD) return false;
-  if (p.K < BKB || (p.K % BKB) != 0) return false;
+  if (p.K < 16 || (p.K & 15) != 0) return false;
+  if (block_scaled && (p.K + BKB - 1) / BKB > 64) return false;  // a tile's weight scales sit in the 64 lanes of one register
   return (int64_t)p.K * 256 < (1ll << 30);
 }
 
