@@ -54,7 +54,9 @@ WORKLOADS = {
 
 
 def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu: int = -1):
-    """Returns (fn, flops_per_step, algorithmic_bytes_per_step, dtype_tag, description, cpu_sample_fn)."""
+    """Returns (fn, flops_per_step, algorithmic_bytes_per_step, dtype_tag, description, cpu_sample_fn); leaves a
+    per-group library-GEMM loop over the same operands in ``build_workload.vendor_loop`` where one exists."""
+    build_workload.vendor_loop = None
     from triton_grouped_gemm_amd import workloads as wl
     from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm_TMA import m_grouped_gemm
     kind, N, K, trans_b = WORKLOADS[name]
@@ -93,6 +95,14 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
                 if t_used >= budget_s:
                     break
             return done_flops / t_used / 1e12, f"{groups} largest groups of {G} ({done_flops / flops * 100:.1f}% of the step's flops), bf16 torch matmul per group"
+        bounds = [(int(s0), int(s0 + n)) for s0, n in zip((sizes_cpu.cumsum(0) - sizes_cpu).tolist(), sizes_cpu.tolist())]
+        c_ref = torch.empty((M_TOTAL, N), device=dev, dtype=torch.bfloat16)
+
+        def vendor_loop():  # one library GEMM per expert, the GPU baseline the reference's tables compare against
+            for g, (s0, s1) in enumerate(bounds):
+                if s1 > s0:
+                    torch.matmul(a[s0:s1], b[g].t() if trans_b else b[g], out=c_ref[s0:s1])
+        build_workload.vendor_loop = vendor_loop
         return fn, flops, nbytes, "bf16", dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, trans_b=trans_b,
                                                group_sizes="dirichlet-multinomial, 128-aligned", seed=seed), cpu_sample
     if kind == "masked":
@@ -113,6 +123,14 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
         a = wl.randn_bf16((M_TOTAL, Md), 1.0, seed + 1, dev)
         b = wl.randn_bf16((M_TOTAL, Nd), 1.0, seed + 2, dev)
         fn = lambda: k_grouped_gemm(a, b, sizes)
+        bounds = [(int(s0), int(s0 + n)) for s0, n in zip((sizes_cpu.cumsum(0) - sizes_cpu).tolist(), sizes_cpu.tolist())]
+        c_ref = torch.zeros((G, Md, Nd), device=dev, dtype=torch.bfloat16)
+
+        def vendor_loop():
+            for g, (s0, s1) in enumerate(bounds):
+                if s1 > s0:
+                    torch.matmul(a[s0:s1].t(), b[s0:s1], out=c_ref[g])
+        build_workload.vendor_loop = vendor_loop
         return (fn, 2.0 * M_TOTAL * Md * Nd, 2.0 * M_TOTAL * (Md + Nd) + 2.0 * G * Md * Nd, "bf16",
                 dict(workload=name, G=G, K_total=M_TOTAL, M_dim=Md, N_dim=Nd, seed=seed), None)
     if kind == "fp8":
@@ -147,6 +165,8 @@ def main() -> int:
     ap.add_argument("--workload", default="bf16_m_grouped_gateup_nt", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="host-core time budget of the CPU baseline sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-vendor-loop", action="store_true",
+                    help="skip timing the per-group torch.matmul (hipBLASLt) loop over the same operands")
     ap.add_argument("--zeros", action="store_true",
                     help="M-grouped bf16 workloads only: all-zero operands (diagnostic: shows how far the clock is held down "
                          "by the power the multipliers draw on random data); reported as data=synthetic-zeros")
@@ -213,6 +233,20 @@ def main() -> int:
                         min_ms=round(min(kernel_ms), 4), avg_ms=round(avg_kernel_ms, 4))
         metric, unit = "quantizer algorithmic GB/s", "GB/s"
 
+    vendor = None
+    if build_workload.vendor_loop is not None and not args.no_vendor_loop:
+        vl = build_workload.vendor_loop
+        vl()
+        torch.cuda.synchronize()
+        n_v = 3
+        tv = time.perf_counter()
+        for _ in range(n_v):
+            vl()
+        torch.cuda.synchronize()
+        v_ms = (time.perf_counter() - tv) * 1e3 / n_v
+        vendor = dict(value=round(flops / (v_ms * 1e-3) / 1e12, 2), unit="TFLOP/s", ms_per_step=round(v_ms, 4),
+                      kind="torch.matmul per group (hipBLASLt), same operands, wall time incl. launches")
+
     cpu_baseline = None
     if cpu_sample is not None and not args.no_cpu_baseline:
         tf, sample = cpu_sample(args.cpu_seconds)
@@ -223,7 +257,7 @@ def main() -> int:
         "metric": metric, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dtype_tag, "data": "synthetic-zeros" if args.zeros else "synthetic", "config": config,
-        "roofline": roofline, "cpu_baseline": cpu_baseline,
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "vendor_loop": vendor,
     }))
     return 0
 
