@@ -97,6 +97,35 @@ int tgg_per_block_cast_to_fp8(const void* x, void* codes, float* scales, int bat
  * `.to(torch.float8_*)` casts of the recipes above). */
 int tgg_cvt_f32_to_fp8(const float* in, void* out, int64_t n, int fmt, void* stream);
 
+/* ---- MoE token permute / unpermute: the steps either side of the grouped GEMMs -----------------------------------
+ * Replace moe_permute_topK_op / moe_recover_topK_op / moe_recover_topK_bwd_op of the reference's baseline extension
+ * (grouped_gemm/csrc/permute.cu:504-690, kernels :40-297; Python side grouped_gemm/grouped_gemm/ops.py:52-257).
+ * dtype codes: 0 bf16, 1 fp16, 2 e4m3fn, 3 e5m2 (row copy only), 4 fp32.  Rows must be multiples of 16 bytes.
+ *
+ * tgg_moe_permute_map: stable sort of the flattened [num_tokens, topk] expert assignment (expert ids in
+ *   [0, num_experts), num_experts <= 1024; an id of -1 marks a dropped assignment).
+ *   row_id_map[k * num_tokens + t] = destination row of assignment (t, k) in expert-major order, ties in flat order
+ *   (what cub::DeviceRadixSort::SortPairs + moe_permute_topK_row_map produce, permute.cu:40-101, :541-548), or -1 when
+ *   dropped or when the destination is >= num_out_tokens (0 = keep all).  tokens_per_expert (optional, int32 or int64
+ *   [num_experts]) receives the per-expert row counts, i.e. the size_per_group argument of the grouped GEMMs.
+ *   workspace: device memory of at least tgg_moe_sort_workspace_bytes(...) bytes, contents irrelevant before and after.
+ * tgg_moe_permute_rows: permuted[row_id_map[k, t], :] = input[t, :] for every kept assignment.
+ * tgg_moe_unpermute: output[t, :] = sum_k probs[t, k] * input[row_id_map[k, t], :] over kept assignments, fp32
+ *   arithmetic, one rounding to the activation type (probs may be null: plain sum; also the backward of permute_rows).
+ * tgg_moe_unpermute_bwd: act_grad[row_id_map[k, t], :] = probs[t, k] * grad_output[t, :];
+ *   prob_grad[t, k] = <grad_output[t, :], fwd_input[row_id_map[k, t], :]> (0 for dropped); prob_grad may be null. */
+int tgg_moe_sort_workspace_bytes(int64_t num_tokens, int topk, int num_experts, int64_t* bytes);
+int tgg_moe_permute_map(const int32_t* indices, int64_t num_tokens, int topk, int num_experts, int64_t num_out_tokens,
+                        int32_t* row_id_map, void* tokens_per_expert, int counts_i64, void* workspace,
+                        int64_t workspace_bytes, void* stream);
+int tgg_moe_permute_rows(const void* input, void* permuted, const int32_t* row_id_map, int64_t num_tokens, int topk,
+                         int hidden, int dtype, void* stream);
+int tgg_moe_unpermute(const void* input, void* output, const int32_t* row_id_map, const float* probs,
+                      int64_t num_tokens, int topk, int hidden, int dtype, void* stream);
+int tgg_moe_unpermute_bwd(const void* grad_output, const void* fwd_input, const int32_t* row_id_map, const float* probs,
+                          void* act_grad, float* prob_grad, int64_t num_tokens, int topk, int hidden, int dtype,
+                          void* stream);
+
 /* Test hook, runs entirely on the host (no GPU needed): the order in which `grid` persistent workgroups walk
  * the output tiles of a launch, computed by the same scheduler functions the kernels execute.  It restates
  * what the reference's grouped_launch / m_indices_pad tile enumeration guarantees

@@ -206,3 +206,33 @@ def test_metrics():
     assert gemm_ref.rdiff(x, x) == 0.0 and gemm_ref.cos_diff(x, x) == pytest.approx(0.0, abs=1e-15)
     assert gemm_ref.rdiff(x, x + torch.tensor([0.0, 0.0, 0.4])) == pytest.approx(0.4 / 4.4)
     assert torch.allclose(gemm_ref.row_max_normalization(torch.tensor([[1.0, -4.0]])), torch.tensor([[0.25, -1.0]]))
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# MoE permute / unpermute oracle: brute force on tiny inputs
+# ---------------------------------------------------------------------------------------------------------------
+def test_permute_oracle_against_brute_force():
+    import torch
+    from oracle import permute_ref
+    indices = torch.tensor([[2, 0], [1, 2], [-1, 0], [2, 1]], dtype=torch.int32)  # 4 tokens, top-2, one dropped
+    x = torch.arange(4 * 3, dtype=torch.float32).reshape(4, 3)
+    # kept assignments in (expert, flat position) order: written out by hand
+    order = [(0, 1), (2, 1), (1, 0), (3, 1), (0, 0), (1, 1), (3, 0)]  # (token, k) for experts 0,0,1,1,2,2,2
+    m = permute_ref.row_id_map(indices)
+    for pos, (t, k) in enumerate(order):
+        assert int(m[k * 4 + t]) == pos
+    assert int(m[0 * 4 + 2]) == -1  # the dropped assignment (token 2, k 0)
+    m5 = permute_ref.row_id_map(indices, 5)
+    assert [int(v) for v in m5] == [v if 0 <= v < 5 else -1 for v in m.tolist()]
+    assert permute_ref.tokens_per_expert(indices, 4).tolist() == [2, 2, 3, 0]
+    # permute / unpermute without drops: a round trip with unit weights multiplies by topk
+    ind2 = torch.tensor([[1, 0], [0, 1], [1, 0]], dtype=torch.int32)
+    xs = torch.arange(3 * 2, dtype=torch.float32).reshape(3, 2) + 1
+    p, so = permute_ref.permute(xs, ind2)
+    assert p.tolist() == [xs[0].tolist(), xs[1].tolist(), xs[2].tolist(), xs[0].tolist(), xs[1].tolist(), xs[2].tolist()]
+    probs = torch.tensor([[0.25, 0.75], [0.5, 0.5], [1.0, 0.0]])
+    u = permute_ref.unpermute(p, so, probs)
+    assert torch.allclose(u, xs * probs.sum(1, keepdim=True))
+    u2 = permute_ref.unpermute(p * torch.tensor([[1.], [1.], [1.], [2.], [2.], [2.]]), so, probs)
+    # expert-1 copies were doubled: token 0 used expert 1 at k=0 (weight .25), token 1 at k=1 (.5), token 2 at k=0 (1.0)
+    assert torch.allclose(u2, xs * torch.tensor([[0.25 * 2 + 0.75], [0.5 + 0.5 * 2], [2.0]]))

@@ -31,6 +31,11 @@ SIGNATURES = {
     "tgg_per_token_cast_to_fp8": [_P, _P, _P, _L, _I, _I, _I, _P],
     "tgg_per_block_cast_to_fp8": [_P, _P, _P, _I, _I, _I, _I, _P],
     "tgg_cvt_f32_to_fp8": [_P, _P, _L, _I, _P],
+    "tgg_moe_sort_workspace_bytes": [_L, _I, _I, _P],
+    "tgg_moe_permute_map": [_P, _L, _I, _I, _L, _P, _P, _I, _P, _L, _P],
+    "tgg_moe_permute_rows": [_P, _P, _P, _L, _I, _I, _I, _P],
+    "tgg_moe_unpermute": [_P, _P, _P, _P, _L, _I, _I, _I, _P],
+    "tgg_moe_unpermute_bwd": [_P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _P],
     "tgg_debug_tile_order": [_P, _I, _I, _L, _L, _I, _I, _I, _I, _P, _L, _P],
     "tgg_set_option": [c_char_p, _I],
     "tgg_version": [],

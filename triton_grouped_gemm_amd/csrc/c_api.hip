@@ -269,6 +269,78 @@ int tgg_cvt_f32_to_fp8(const float* in, void* out, int64_t n, int fmt, void* str
   return launch_cvt_fp8(in, out, n, fmt, (hipStream_t)stream);
 }
 
+// ---- MoE permute / unpermute ----------------------------------------------------------------------------------
+static int moe_row_bytes(int hidden, int dtype, int64_t* row_bytes) {
+  int esz;
+  if (dtype == DT_BF16 || dtype == DT_F16) esz = 2;
+  else if (dtype == DT_E4M3 || dtype == DT_E5M2) esz = 1;
+  else if (dtype == 4) esz = 4;
+  else return set_error("unsupported activation dtype code %d", dtype);
+  if (hidden < 1) return set_error("hidden size must be positive");
+  *row_bytes = (int64_t)hidden * esz;
+  if (*row_bytes % 16 != 0) return set_error("rows must be a multiple of 16 bytes (hidden=%d, %d-byte elements)", hidden, esz);
+  return 0;
+}
+
+int tgg_moe_sort_workspace_bytes(int64_t num_tokens, int topk, int num_experts, int64_t* bytes) {
+  if (!bytes) return set_error("null pointer");
+  if (num_tokens < 0 || topk < 1) return set_error("bad num_tokens / topk");
+  if (num_experts < 1 || num_experts > 1024) return set_error("num_experts=%d outside [1, 1024]", num_experts);
+  *bytes = moe_sort_workspace_bytes(num_tokens * topk, num_experts);
+  return 0;
+}
+
+int tgg_moe_permute_map(const int32_t* indices, int64_t num_tokens, int topk, int num_experts, int64_t num_out_tokens,
+                        int32_t* row_id_map, void* tokens_per_expert, int counts_i64, void* workspace,
+                        int64_t workspace_bytes, void* stream) {
+  if (num_tokens < 0 || topk < 1) return set_error("bad num_tokens / topk");
+  if (num_tokens * topk >= (1ll << 31)) return set_error("num_tokens * topk must stay below 2^31");
+  if (num_experts < 1 || num_experts > 1024) return set_error("num_experts=%d outside [1, 1024]", num_experts);
+  if (!workspace || (num_tokens > 0 && (!indices || !row_id_map))) return set_error("null pointer");
+  if (workspace_bytes < moe_sort_workspace_bytes(num_tokens * topk, num_experts))
+    return set_error("workspace of %lld bytes is too small (need %lld)", (long long)workspace_bytes,
+                     (long long)moe_sort_workspace_bytes(num_tokens * topk, num_experts));
+  const int64_t capacity = num_out_tokens > 0 ? num_out_tokens : num_tokens * topk;
+  return launch_moe_permute_map(indices, num_tokens, topk, num_experts, capacity, row_id_map, tokens_per_expert,
+                                counts_i64, workspace, (hipStream_t)stream);
+}
+
+int tgg_moe_permute_rows(const void* input, void* permuted, const int32_t* row_id_map, int64_t num_tokens, int topk,
+                         int hidden, int dtype, void* stream) {
+  int64_t rb;
+  if (moe_row_bytes(hidden, dtype, &rb)) return 1;
+  if (num_tokens < 0 || topk < 1) return set_error("bad num_tokens / topk");
+  if (num_tokens > 0 && (!input || !permuted || !row_id_map)) return set_error("null pointer");
+  if (!aligned16(input) || !aligned16(permuted)) return set_error("activation pointers must be 16-byte aligned");
+  return launch_moe_permute_rows(input, permuted, row_id_map, num_tokens, topk, rb, (hipStream_t)stream);
+}
+
+int tgg_moe_unpermute(const void* input, void* output, const int32_t* row_id_map, const float* probs,
+                      int64_t num_tokens, int topk, int hidden, int dtype, void* stream) {
+  int64_t rb;
+  if (moe_row_bytes(hidden, dtype, &rb)) return 1;
+  if (dtype == DT_E4M3 || dtype == DT_E5M2) return set_error("unpermute computes in fp32 on bf16 / fp16 / fp32 rows only");
+  if (num_tokens < 0 || topk < 1) return set_error("bad num_tokens / topk");
+  if (num_tokens > 0 && (!input || !output || !row_id_map)) return set_error("null pointer");
+  if (!aligned16(input) || !aligned16(output)) return set_error("activation pointers must be 16-byte aligned");
+  return launch_moe_unpermute(input, output, row_id_map, probs, num_tokens, topk, rb, dtype, (hipStream_t)stream);
+}
+
+int tgg_moe_unpermute_bwd(const void* grad_output, const void* fwd_input, const int32_t* row_id_map, const float* probs,
+                          void* act_grad, float* prob_grad, int64_t num_tokens, int topk, int hidden, int dtype,
+                          void* stream) {
+  int64_t rb;
+  if (moe_row_bytes(hidden, dtype, &rb)) return 1;
+  if (dtype == DT_E4M3 || dtype == DT_E5M2) return set_error("unpermute computes in fp32 on bf16 / fp16 / fp32 rows only");
+  if (num_tokens < 0 || topk < 1) return set_error("bad num_tokens / topk");
+  if (num_tokens > 0 && (!grad_output || !act_grad || !row_id_map)) return set_error("null pointer");
+  if (prob_grad && (!probs || !fwd_input)) return set_error("prob_grad needs probs and the forward input");
+  if (!aligned16(grad_output) || !aligned16(act_grad) || !aligned16(fwd_input))
+    return set_error("activation pointers must be 16-byte aligned");
+  return launch_moe_unpermute_bwd(grad_output, fwd_input, row_id_map, probs, act_grad, prob_grad, num_tokens, topk, rb,
+                                  dtype, (hipStream_t)stream);
+}
+
 int tgg_debug_tile_order(const int64_t* sizes, int G, int mode, int64_t m_total, int64_t aux, int N, int tile,
                          int grid, int split, int64_t* out, int64_t capacity, int64_t* num_tiles) {
   if (!sizes || !out || !num_tiles) return set_error("null pointer");
