@@ -135,15 +135,34 @@ __global__ __launch_bounds__(256) void trans_quant128_kernel(const uint16_t* __r
   }
 }
 
-// 16 lanes per 1x128 group; each lane 8 elements.
+// 16 lanes per 1x128 group; each lane 8 elements.  A workgroup's 16 lane groups take 16 neighbouring groups
+// along the axis the scales are contiguous in, so that the 16 scale stores of a step fill one 64-byte segment:
+//   scales [rows, kblocks]  (mn_major = 0): 16 consecutive K blocks of one row
+//   scales [kblocks, rows]  (mn_major = 1): the same K block of 16 consecutive rows
+// Two steps are in flight per thread.
 template <int FMT>
 __global__ __launch_bounds__(256) void token_cast128_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ codes,
                                                            float* __restrict__ scales, int64_t rows, int kblocks, int mn_major) {
   constexpr float fmax_ = FmtMax<FMT>::v;
   const int64_t groups = rows * kblocks;
-  const int sub = threadIdx.x & 15;
-  for (int64_t g = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4); g < groups; g += (int64_t)gridDim.x * 16) {
-    const i32x4_t v = *(const i32x4_t*)(x + g * 128 + sub * 8);
+  const int sub = threadIdx.x & 15, grp = threadIdx.x >> 4;
+  // step s of the launch covers 16 groups; steps are numbered so that consecutive steps touch neighbouring memory
+  const int64_t row_blocks = (rows + 15) / 16;
+  const int64_t steps = mn_major ? row_blocks * kblocks : (groups + 15) / 16;
+  auto group_of = [&](int64_t step, int64_t& g, int64_t& sidx) -> bool {
+    if (mn_major) {
+      const int64_t rb = step / kblocks;
+      const int kb = (int)(step - rb * kblocks);
+      const int64_t r = rb * 16 + grp;
+      g = r * kblocks + kb;
+      sidx = (int64_t)kb * rows + r;
+      return r < rows;
+    }
+    g = step * 16 + grp;
+    sidx = g;
+    return g < groups;
+  };
+  auto quantise = [&](const i32x4_t v, int64_t g, int64_t sidx, bool ok) {
     float amax = amax8(v);
 #pragma unroll
     for (int off = 8; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
@@ -159,8 +178,20 @@ __global__ __launch_bounds__(256) void token_cast128_kernel(const uint16_t* __re
     uint2 pk;
     pk.x = cvt4<FMT>(f[0], f[1], f[2], f[3]);
     pk.y = cvt4<FMT>(f[4], f[5], f[6], f[7]);
-    *(uint2*)(codes + g * 128 + sub * 8) = pk;
-    if (sub == 0) scales[mn_major ? (g % kblocks) * rows + g / kblocks : g] = amax / fmax_;
+    if (ok) {
+      *(uint2*)(codes + g * 128 + sub * 8) = pk;
+      if (sub == 0) scales[sidx] = amax / fmax_;
+    }
+  };
+  const i32x4_t zero = {0, 0, 0, 0};
+  for (int64_t s0 = (int64_t)blockIdx.x * 2; s0 < steps; s0 += (int64_t)gridDim.x * 2) {
+    int64_t g0, g1, i0, i1;
+    const bool ok0 = group_of(s0, g0, i0);
+    const bool ok1 = s0 + 1 < steps && group_of(s0 + 1, g1, i1);
+    const i32x4_t v0 = ok0 ? *(const i32x4_t*)(x + g0 * 128 + sub * 8) : zero;
+    const i32x4_t v1 = ok1 ? *(const i32x4_t*)(x + g1 * 128 + sub * 8) : zero;
+    quantise(v0, g0, i0, ok0);
+    quantise(v1, g1, i1, ok1);
   }
 }
 
@@ -263,7 +294,7 @@ int launch_token_cast128(const void* x, void* codes, float* scales, int64_t rows
                          hipStream_t s) {
   const int64_t groups = rows * kblocks;
   if (groups == 0) return 0;
-  int64_t grid = (groups + 15) / 16;
+  int64_t grid = ((mn_major ? ((rows + 15) / 16) * kblocks : (groups + 15) / 16) + 1) / 2;
   const int64_t cap = (int64_t)num_cus() * 32;
   if (grid > cap) grid = cap;
   if (fmt == DT_E4M3)
