@@ -52,8 +52,8 @@ TGG_DEV float amax8(i32x4_t v) {
   return m;
 }
 
-struct TransSmem {
-  SchedTable sched;
+template <int MAXG> struct TransSmem {
+  SchedTableT<MAXG> sched;
   __attribute__((aligned(16))) uint8_t t[128 * 128];
   float wmax[4];
 };
@@ -61,10 +61,11 @@ struct TransSmem {
 // One 128x128 block per iteration, 256 threads.
 // Read: thread (rr = tid/16, cv = tid%16) owns rows rr*8 .. rr*8+7, columns cv*8 .. cv*8+7.
 // LDS holds the transposed codes: byte (c, r) at c*128 + ((r/16) ^ ((c/8)%8))*16 + r%16.
-template <int FMT>
+// MAXG sizes the group table in LDS: the small one lets twice as many workgroups share a CU.
+template <int FMT, int MAXG>
 __global__ __launch_bounds__(256) void trans_quant128_kernel(const uint16_t* __restrict__ x, uint8_t* __restrict__ codes,
                                                             float* __restrict__ scales, GemmParams p, int64_t m_expand) {
-  __shared__ TransSmem sm;
+  __shared__ TransSmem<MAXG> sm;
   sched_init<128>(p, sm.sched);
   const int N = p.N;
   const int tiles_n = N >> 7;
@@ -279,14 +280,19 @@ int launch_trans_quant128(const void* x, void* codes, float* scales, const GemmP
   int64_t grid = (int64_t)num_cus() * 8;
   if (grid > tiles) grid = tiles;
   if (grid < 1) grid = 1;
-  if (fmt == DT_E4M3)
-    hipLaunchKernelGGL(trans_quant128_kernel<DT_E4M3>, dim3((unsigned)grid), dim3(256), 0, s, (const uint16_t*)x,
-                       (uint8_t*)codes, scales, p, m_expand);
-  else if (fmt == DT_E5M2)
-    hipLaunchKernelGGL(trans_quant128_kernel<DT_E5M2>, dim3((unsigned)grid), dim3(256), 0, s, (const uint16_t*)x,
-                       (uint8_t*)codes, scales, p, m_expand);
-  else
+  const dim3 g((unsigned)grid), b(256);
+  const uint16_t* xi = (const uint16_t*)x;
+  uint8_t* co = (uint8_t*)codes;
+  const bool small = p.G <= 256;
+  if (fmt == DT_E4M3) {
+    if (small) hipLaunchKernelGGL((trans_quant128_kernel<DT_E4M3, 256>), g, b, 0, s, xi, co, scales, p, m_expand);
+    else hipLaunchKernelGGL((trans_quant128_kernel<DT_E4M3, kMaxGroups>), g, b, 0, s, xi, co, scales, p, m_expand);
+  } else if (fmt == DT_E5M2) {
+    if (small) hipLaunchKernelGGL((trans_quant128_kernel<DT_E5M2, 256>), g, b, 0, s, xi, co, scales, p, m_expand);
+    else hipLaunchKernelGGL((trans_quant128_kernel<DT_E5M2, kMaxGroups>), g, b, 0, s, xi, co, scales, p, m_expand);
+  } else {
     return set_error("unsupported fp8 format code %d", fmt);
+  }
   return check_launch("trans_quant128");
 }
 
