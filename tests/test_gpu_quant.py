@@ -42,6 +42,7 @@ def test_hardware_fp8_conversion_equals_software_rne(dev, fmt, code):
     ([5, 0, 130, 128, 1], 256),
     ([0, 0, 0], 128),
     ([300] * 7 + [77], 384),
+    ([3, 0, 17] * 100, 128),  # 300 groups: the large group table
 ])
 def test_trans_quant_bit_exact(dev, dtype, sizes, N):
     M = sum(sizes)
