@@ -218,3 +218,17 @@ def test_medium_dirichlet_config_shape(dev, variant):
         n = min(n, 512)
         ag = a[s0:s0 + n]
         check_16bit_gemm(out[s0:s0 + n], ag @ b[g].t(), ag.float() @ b[g].float().t(), f"medium g{g}")
+
+
+@pytest.mark.parametrize("G", [384, 512, 600])  # up to 512 groups run on the tuned kernels, more on the shape-agnostic one
+def test_many_groups_exact(dev, variant, G):
+    pattern = [3, 0, 70, 129, 1, 256]
+    sizes = [pattern[g % len(pattern)] for g in range(G)]
+    M, N, K = sum(sizes), 136, 64
+    a = _ints((M, K), 21, torch.bfloat16)
+    b = _ints((G, N, K), 22, torch.bfloat16)
+    out = m_grouped_gemm(a.to(dev), b.to(dev), torch.tensor(sizes, dtype=torch.int32, device=dev), True)
+    assert torch.equal(out.cpu(), gemm_ref.gmm_fp32(a, b, sizes, True).to(torch.bfloat16))
+    kt = k_grouped_gemm(a.to(dev), a.to(dev), torch.tensor(sizes, dtype=torch.int64, device=dev))
+    ref = gemm_ref.gmm_dw(a, a, sizes, fp32=True)
+    assert ref.abs().max() <= 256 and torch.equal(kt.cpu(), ref.to(torch.bfloat16))

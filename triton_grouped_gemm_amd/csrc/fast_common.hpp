@@ -42,7 +42,7 @@ TGG_DEV i32x4_t make_rsrc(uint64_t base, int64_t bytes) {
   return r;
 }
 
-constexpr int kFastMaxGroups = 256;
+constexpr int kFastMaxGroups = 512;
 constexpr int kSlabRowBytes = 128;  // a slab holds 128 bytes of every K-contiguous row (64 bf16 / 128 fp8 values)
 
 // Geometry of one operand's slab in LDS and of the copies that fill it.
