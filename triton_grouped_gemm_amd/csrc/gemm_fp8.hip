@@ -190,8 +190,6 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
     }
   };
 
-  char* const stage_c = smem + C::EPI_OFF + wave * C::EPI_WAVE_BYTES;
-
   // Software pipeline.  A slab is worked off in TM x 2 cells (32-row block i, 32-column block j), two
   // 64-deep multiplies each.  The B fragments of both column blocks stay in registers for the slab, the
   // A fragments of row block i+1 are read during row block i.  Before the last cell (TM-1, 1): wait for
@@ -312,16 +310,38 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
     }
 
     // Epilogue (see gemm_fast.hip): per-channel scaling happens on the fp32 values before packing.
+    // The lane id passes through an opaque statement so that the address arithmetic below is redone per tile
+    // instead of being hoisted: hoisted values would have to live (spilled) across the register-tight main loop,
+    // and every reload waits for all outstanding stores.
+    int el = lane;
+    asm volatile("" : "+v"(el));
+    const int e32 = el & 31, eh = el >> 5;
+    const int st_row = el >> 2, st_chunk = el & 3;
+    char* const stage = smem + C::EPI_OFF + wave * C::EPI_WAVE_BYTES;
     const int64_t c_row0 = KGROUP ? ((int64_t)cur.g * p.m_total + cur.row0) : cur.row0;
     char* const c_tile = (char*)p.C + ((c_row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2;
-    const int st_row = lane >> 2, st_chunk = lane & 3;
+    // channel scales of this lane's rows and columns, fetched up front in a few wide loads
+    float rs[C::TM];
+    f32x4_t cs[C::TN][4];
+    if (EPI == EPI_CHANNEL) {
+      const float* sm = p.scale_m + (KGROUP ? (int64_t)cur.g * p.scale_m_sg : 0) + cur.row0;
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i) {
+        const int m = wm0 + 32 * i + e32;
+        rs[i] = m < cur.rows ? sm[m] : 0.f;
+      }
+      const float* sn = p.scale_n + (int64_t)cur.g * p.N;
+#pragma unroll
+      for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = cur.n0 + wn0 + 32 * j + 8 * q + 4 * eh;  // N is a multiple of 8: 4 columns are in or out together
+          const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+          cs[j][q] = n < p.N ? *(const f32x4_t*)(sn + n) : zero;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < C::TM; ++i) {
-      float rs = 1.f;
-      if (EPI == EPI_CHANNEL) {
-        const int m = wm0 + 32 * i + l32;
-        rs = m < cur.rows ? p.scale_m[(KGROUP ? (int64_t)cur.g * p.scale_m_sg : 0) + cur.row0 + m] : 0.f;
-      }
 #pragma unroll
       for (int j = 0; j < C::TN; ++j) {
 #pragma unroll
@@ -330,17 +350,16 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
           if (EPI == EPI_CHANNEL) {
-            const int n = cur.n0 + wn0 + 32 * j + 8 * q + 4 * lh;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = (n + e < p.N) ? v[e] * rs * p.scale_n[(int64_t)cur.g * p.N + n + e] : 0.f;
+            for (int e = 0; e < 4; ++e) v[e] = v[e] * rs[i] * cs[j][q][e];
           }
-          *(uint2*)(stage_c + l32 * C::EPI_PITCH + (8 * q + 4 * lh) * 2) = pack4<OUT>(v[0], v[1], v[2], v[3]);
+          *(uint2*)(stage + e32 * C::EPI_PITCH + (8 * q + 4 * eh) * 2) = pack4<OUT>(v[0], v[1], v[2], v[3]);
         }
         const bool col_ok = cur.n0 + wn0 + 32 * j + st_chunk * 8 < p.N;
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
           const int r = it * 16 + st_row;
-          const i32x4_t v = *(const i32x4_t*)(stage_c + r * C::EPI_PITCH + st_chunk * 16);
+          const i32x4_t v = *(const i32x4_t*)(stage + r * C::EPI_PITCH + st_chunk * 16);
           if (col_ok && wm0 + 32 * i + r < cur.rows)
             *(i32x4_t*)(c_tile + ((int64_t)(32 * i + r) * p.N + 32 * j + st_chunk * 8) * 2) = v;
         }
