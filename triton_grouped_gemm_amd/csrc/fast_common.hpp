@@ -42,6 +42,16 @@ TGG_DEV i32x4_t make_rsrc(uint64_t base, int64_t bytes) {
   return r;
 }
 
+// The same with a 32-bit length (negative = nothing left).
+TGG_DEV i32x4_t make_rsrc32(uint64_t base, int bytes) {
+  i32x4_t r;
+  r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)base);
+  r[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(base >> 32) & 0xffff);  // stride 0, no swizzle
+  r[2] = __builtin_amdgcn_readfirstlane(bytes < 0 ? 0 : bytes);
+  r[3] = 0x00020000;  // 32-bit data format
+  return r;
+}
+
 constexpr int kFastMaxGroups = 512;
 constexpr int kSlabRowBytes = 128;  // a slab holds 128 bytes of every K-contiguous row (64 bf16 / 128 fp8 values)
 

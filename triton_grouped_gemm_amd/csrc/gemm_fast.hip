@@ -160,11 +160,15 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
     }
   };
 
-  // Slab sequence of a tile, held in scalar registers: where the next slab of each operand starts, how
-  // many bytes may still be touched from there (everything beyond reads as zero), how many slabs exist.
+  // Slab sequence of a tile, held in scalar registers: where the next slab of each operand starts and how far
+  // the copies may reach from there (everything beyond reads as zero).  32-bit bookkeeping keeps the per-slab
+  // scalar work short (eight waves share the CU's scalar unit):
+  //   K-contiguous operand  rem = bytes left in the tile's window of rows (it shrinks by 128 per slab)
+  //   token-row operand     rem = token rows left in the reduction range; a slab may touch
+  //                         min(rem, BK) * row pitch - off bytes, off = byte offset of the tile inside a row
   struct TileIo {
     uint64_t a_base, b_base;
-    int64_t a_left, b_left;
+    int a_rem, b_rem, a_off, b_off;
     int kt_n, issued;
   };
   const int64_t a_step = A_KMAJOR ? BK * 2 : BK * a_ld;
@@ -175,29 +179,35 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   auto make_io = [&](const Tile& t) {
     TileIo io;
     io.kt_n = slabs_of(t);
+    io.a_off = io.b_off = 0;
     if (LAYOUT == LAYOUT_TN) {
-      const int64_t klen = t.k1 - t.k0;
+      const int klen = (int)(t.k1 - t.k0);
       io.a_base = (uint64_t)p.A + (uint64_t)(t.k0 * a_ld + t.row0 * 2);
-      io.a_left = klen * a_ld - t.row0 * 2;
+      io.a_rem = klen;
+      io.a_off = (int)(t.row0 * 2);
       io.b_base = (uint64_t)p.B + (uint64_t)(t.k0 * b_ld + (int64_t)t.n0 * 2);
-      io.b_left = klen * b_ld - (int64_t)t.n0 * 2;
+      io.b_rem = klen;
+      io.b_off = t.n0 * 2;
     } else {
       const int64_t rows_left = p.m_total - t.row0;
       io.a_base = (uint64_t)p.A + (uint64_t)(t.row0 * a_ld);
-      io.a_left = (rows_left < C::BM ? rows_left : C::BM) * a_ld;
+      io.a_rem = (int)(rows_left < C::BM ? rows_left : C::BM) * (int)a_ld;
       if (LAYOUT == LAYOUT_NT) {
         const int n_left = p.N - t.n0;
         io.b_base = (uint64_t)p.B + (uint64_t)(((int64_t)t.g * p.N + t.n0) * b_ld);
-        io.b_left = (int64_t)(n_left < C::BN ? n_left : C::BN) * b_ld;
+        io.b_rem = (n_left < C::BN ? n_left : C::BN) * (int)b_ld;
       } else {
         io.b_base = (uint64_t)p.B + (uint64_t)((int64_t)t.g * p.K * b_ld + (int64_t)t.n0 * 2);
-        io.b_left = (int64_t)p.K * b_ld - (int64_t)t.n0 * 2;
+        io.b_rem = p.K;
+        io.b_off = t.n0 * 2;
       }
     }
     io.a_base = uniform64(io.a_base);
     io.b_base = uniform64(io.b_base);
-    io.a_left = (int64_t)uniform64((uint64_t)io.a_left);
-    io.b_left = (int64_t)uniform64((uint64_t)io.b_left);
+    io.a_rem = __builtin_amdgcn_readfirstlane(io.a_rem);
+    io.b_rem = __builtin_amdgcn_readfirstlane(io.b_rem);
+    io.a_off = __builtin_amdgcn_readfirstlane(io.a_off);
+    io.b_off = __builtin_amdgcn_readfirstlane(io.b_off);
     io.kt_n = __builtin_amdgcn_readfirstlane(io.kt_n);
     io.issued = 0;
     return io;
@@ -215,7 +225,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
     feed.kt_n = 0;
     feed.issued = 0;
     feed.a_base = feed.b_base = (uint64_t)p.A;
-    feed.a_left = feed.b_left = 0;
+    feed.a_rem = feed.b_rem = feed.a_off = feed.b_off = 0;
     for (; id < walk.end; id += walk.stride) {
       const Tile tt = sched_tile<C::BM, C::BN>(p, sched, id);
       if (slabs_of(tt) > 0) {
@@ -238,14 +248,16 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   auto begin_slab = [&](int buf) {
     SlabCopy sc;
     const bool live = feed.issued < feed.kt_n;
-    sc.ra = make_rsrc(feed.a_base, live ? feed.a_left : 0);
-    sc.rb = make_rsrc(feed.b_base, live ? feed.b_left : 0);
+    const int a_len = A_KMAJOR ? feed.a_rem : min(feed.a_rem, BK) * (int)a_ld - feed.a_off;
+    const int b_len = B_KMAJOR ? feed.b_rem : min(feed.b_rem, BK) * (int)b_ld - feed.b_off;
+    sc.ra = make_rsrc32(feed.a_base, live ? a_len : 0);
+    sc.rb = make_rsrc32(feed.b_base, live ? b_len : 0);
     sc.base = smem_addr + buf * C::STAGE_BYTES;
     sc.tail = tail_chunks != 0 && feed.issued + 1 == feed.kt_n;
     feed.a_base += a_step;
-    feed.a_left -= a_step;
+    feed.a_rem -= A_KMAJOR ? BK * 2 : BK;
     feed.b_base += b_step;
-    feed.b_left -= b_step;
+    feed.b_rem -= B_KMAJOR ? BK * 2 : BK;
     feed.issued += 1;
     if (live && feed.issued >= feed.kt_n) feed_seek(feed_id + walk.stride);
     return sc;
@@ -301,8 +313,9 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
     // One K step: multiply (fa, fb); right after the first multiply, read the fragments of K step ks_next
     // of the slab at s_next into (fna, fnb); copies [k0, k0 + NC/2) of `sc` are issued one per SP
     // multiplies when k0 >= 0.
+    SlabCopy sc_next;
     auto step = [&](const i32x4_t (&fa)[C::TM], const i32x4_t (&fb)[C::TN], const char* s_next, int ks_next,
-                    i32x4_t (&fna)[C::TM], i32x4_t (&fnb)[C::TN], int k0) {
+                    i32x4_t (&fna)[C::TM], i32x4_t (&fnb)[C::TN], int k0, bool prepare = false) {
 #pragma unroll
       for (int i = 0; i < C::TM; ++i)
 #pragma unroll
@@ -314,6 +327,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
             load_frags(s_next, ks_next, fna, fnb);
             __builtin_amdgcn_sched_barrier(0);
           }
+          if (prepare && n == 1) sc_next = begin_slab(ring & 1);  // scalar work, under the multiplies just issued
           if (k0 >= 0 && (n + 1) % SP == 0 && (n + 1) / SP <= NC / 2) {
             __builtin_amdgcn_sched_barrier(0);
             copy_k(sc, k0 + (n + 1) / SP - 1);
@@ -328,8 +342,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
       const char* sn = smem + ((ring + 1) & 1) * C::STAGE_BYTES;
       step(fa0, fb0, sa, 1, fa1, fb1, NC / 2);
       step(fa1, fb1, sa, 2, fa0, fb0, -1);
-      step(fa0, fb0, sa, 3, fa1, fb1, -1);
-      const SlabCopy sc_next = begin_slab(ring & 1);  // scalar work only: overlaps the multiplies in flight
+      step(fa0, fb0, sa, 3, fa1, fb1, -1, true);
       wait_vmcnt<0>();
       __syncthreads();
       sc = sc_next;

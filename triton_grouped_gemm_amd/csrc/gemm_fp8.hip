@@ -100,7 +100,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
   // of A, B and (block scaling) of the tile rows' activation scales, which are stored [K/128, m_total].
   struct TileIo {
     uint64_t a_base, b_base, s_base;
-    int64_t a_left, b_left;
+    int a_left, b_left;  // operand windows stay below 2^30 bytes: 32-bit scalar bookkeeping
     int s_bytes, kt_n, issued;
   };
   auto slabs_of = [&](const Tile& t) -> int { return KGROUP ? (int)((t.k1 - t.k0 + BKB - 1) / BKB) : (p.K + BKB - 1) / BKB; };
@@ -112,9 +112,9 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
     const int a_rows = (int)(rows_left < C::BM ? rows_left : C::BM);
     const int n_left = p.N - t.n0;
     io.a_base = uniform64((uint64_t)p.A + (uint64_t)(t.row0 * ld + k0));
-    io.a_left = (int64_t)uniform64((uint64_t)((int64_t)a_rows * ld - k0));
+    io.a_left = __builtin_amdgcn_readfirstlane((int)((int64_t)a_rows * ld - k0));
     io.b_base = uniform64((uint64_t)p.B + (uint64_t)((KGROUP ? (int64_t)t.n0 : ((int64_t)t.g * p.N + t.n0)) * ld + k0));
-    io.b_left = (int64_t)uniform64((uint64_t)((int64_t)(n_left < C::BN ? n_left : C::BN) * ld - k0));
+    io.b_left = __builtin_amdgcn_readfirstlane((int)((int64_t)(n_left < C::BN ? n_left : C::BN) * ld - k0));
     io.s_base = BLOCK ? uniform64((uint64_t)(p.sa + t.row0)) : 0;
     io.s_bytes = BLOCK ? __builtin_amdgcn_readfirstlane(a_rows * 4) : 0;
     io.issued = 0;
@@ -160,9 +160,9 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
   auto begin_slab = [&](int buf) {
     SlabCopy sc;
     const bool live = feed.issued < feed.kt_n;
-    sc.ra = make_rsrc(feed.a_base, live ? feed.a_left : 0);
-    sc.rb = make_rsrc(feed.b_base, live ? feed.b_left : 0);
-    sc.rs = make_rsrc(feed.s_base, live ? feed.s_bytes : 0);
+    sc.ra = make_rsrc32(feed.a_base, live ? feed.a_left : 0);
+    sc.rb = make_rsrc32(feed.b_base, live ? feed.b_left : 0);
+    sc.rs = make_rsrc32(feed.s_base, live ? feed.s_bytes : 0);
     sc.base = smem_addr + buf * C::STAGE_BYTES;
     sc.tail = tail_chunks != 0 && feed.issued + 1 == feed.kt_n;
     feed.a_base += BKB;
@@ -294,8 +294,8 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
           cell(i + 1, 0, 6 + 4 * i, fay, fb0, [&] { load_frag(sa + (wm0 + 32 * (i + 2)) * 128, fax); });
           cell(i + 1, 1, 8 + 4 * i, fay, fb1, [&] {});
         } else {
-          cell(i + 1, 0, 6 + 4 * i, fay, fb0, [&] {});
-          const SlabCopy scn = begin_slab(ring & 1);  // scalar work only: overlaps the multiplies in flight
+          SlabCopy scn;
+          cell(i + 1, 0, 6 + 4 * i, fay, fb0, [&] { scn = begin_slab(ring & 1); });  // scalar work under a multiply
           wait_vmcnt<0>();
           if (BLOCK) asm volatile("" : "+v"(sbv_next));  // nothing of this wave is in flight: touching it costs no wait
           __syncthreads();
