@@ -48,6 +48,7 @@ WORKLOADS = {
     "bf16_m_grouped_gateup_nn": ("mg", 1536, 2048, False),
     "bf16_m_grouped_down_nt": ("mg", 2048, 768, True),
     "bf16_m_grouped_down_nn": ("mg", 2048, 768, False),
+    "bf16_m_grouped_gateup_fp8_out": ("mgq", 1536, 2048, True),   # same GEMM, output quantised 1x128 in the epilogue
     "bf16_masked_decode": ("masked", 4096, 1536, True),
     "bf16_k_grouped_wgrad": ("kg", 4096, 3072, False),      # N_DIM, M_DIM
     "fp8_block_m_grouped": ("fp8", 3072, 4096, True),
@@ -110,6 +111,15 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
         build_workload.vendor_loop = vendor_loop
         return fn, flops, nbytes, "bf16", dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, trans_b=trans_b,
                                                group_sizes="dirichlet-multinomial, 128-aligned", seed=seed), cpu_sample
+    if kind == "mgq":
+        from triton_grouped_gemm_amd.gemm.fused import m_grouped_gemm_fp8_out
+        a = wl.randn_bf16((M_TOTAL, K), K ** -0.5, seed + 1, dev)
+        b = wl.randn_bf16((G, N, K), K ** -0.5, seed + 2, dev)
+        fn = lambda: m_grouped_gemm_fp8_out(a, b, sizes, trans_b, scales_mn_major=True)
+        nbytes = 2.0 * M_TOTAL * K + 2.0 * G * N * K + 1.0 * M_TOTAL * N + 4.0 * M_TOTAL * N / 128
+        return (fn, 2.0 * M_TOTAL * N * K, nbytes, "bf16",
+                dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, trans_b=trans_b, output="e4m3fn codes + 1x128 fp32 scales",
+                     group_sizes="dirichlet-multinomial, 128-aligned", seed=seed), None)
     if kind == "masked":
         from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm_masked_TMA import m_grouped_gemm_masked
         m_max = 512

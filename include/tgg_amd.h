@@ -97,6 +97,18 @@ int tgg_per_block_cast_to_fp8(const void* x, void* codes, float* scales, int bat
  * `.to(torch.float8_*)` casts of the recipes above). */
 int tgg_cvt_f32_to_fp8(const float* in, void* out, int64_t n, int fmt, void* stream);
 
+/* M-grouped GEMM whose output leaves as FP8 codes with one fp32 scale per row and 128 columns (the 1x128 activation
+ * recipe), bit-identical to tgg_m_grouped_gemm followed by tgg_per_token_cast_to_fp8 on its 16-bit result but without
+ * the round trip through memory.  codes [M, N] fp8 (fmt 2 = e4m3fn, 3 = e5m2); scales [M, N/128] fp32, or stored
+ * [N/128, M] when scales_mn_major (what the block-scaled GEMM consumes).  N must be a multiple of 128.  Returns 1 with
+ * a message for shapes the fused kernel does not take (more than 512 groups, very long rows); the two separate calls
+ * give the same result.  No counterpart in the reference's Python API: it fuses m_grouped_gemm
+ * (gemm/BF16/m_grouped_gemm_TMA.py:435) with per_token_cast_to_fp8 (gemm/FP8/m_grouped_gemm_channel_expert.py:217-222),
+ * the step between the two expert GEMMs of an FP8 MoE layer. */
+int tgg_m_grouped_gemm_fp8_out(const void* A, const void* B, void* codes, float* scales, const void* sizes,
+                               int sizes_i64, int G, int64_t M, int N, int K, int trans_b, int dtype, int fmt,
+                               int scales_mn_major, int num_cu, void* stream);
+
 /* ---- MoE token permute / unpermute: the steps either side of the grouped GEMMs -----------------------------------
  * Replace moe_permute_topK_op / moe_recover_topK_op / moe_recover_topK_bwd_op of the reference's baseline extension
  * (grouped_gemm/csrc/permute.cu:504-690, kernels :40-297; Python side grouped_gemm/grouped_gemm/ops.py:52-257).

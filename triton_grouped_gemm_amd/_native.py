@@ -31,6 +31,7 @@ SIGNATURES = {
     "tgg_per_token_cast_to_fp8": [_P, _P, _P, _L, _I, _I, _I, _P],
     "tgg_per_block_cast_to_fp8": [_P, _P, _P, _I, _I, _I, _I, _P],
     "tgg_cvt_f32_to_fp8": [_P, _P, _L, _I, _P],
+    "tgg_m_grouped_gemm_fp8_out": [_P, _P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _I, _I, _I, _P],
     "tgg_moe_sort_workspace_bytes": [_L, _I, _I, _P],
     "tgg_moe_permute_map": [_P, _L, _I, _I, _L, _P, _P, _I, _P, _L, _P],
     "tgg_moe_permute_rows": [_P, _P, _P, _L, _I, _I, _I, _P],

@@ -49,6 +49,8 @@ int launch_block_cast128(const void*, void*, float*, int, int, int, int, hipStre
 int launch_cvt_fp8(const float*, void*, int64_t, int, hipStream_t);
 bool fast_supported(const GemmParams& p, int dt, int layout);
 int launch_fast_16bit(const GemmParams& p, int dt, int layout, hipStream_t s);
+bool fast_quant_supported(const GemmParams& p, int dt, int layout);
+int launch_fast_16bit_quant(const GemmParams& p, int dt, int layout, hipStream_t s);
 void set_fast_variant(int v);
 
 static bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
@@ -122,6 +124,33 @@ int tgg_m_grouped_gemm(const void* A, const void* B, void* C, const void* sizes,
   if (trans_b) { p.b_sn = K; p.b_sk = 1; } else { p.b_sn = 1; p.b_sk = N; }
   p.grid_limit = num_cu;
   return dispatch_16bit(p, dtype, trans_b ? 0 : 1, (hipStream_t)stream);
+}
+
+int tgg_m_grouped_gemm_fp8_out(const void* A, const void* B, void* codes, float* scales, const void* sizes,
+                               int sizes_i64, int G, int64_t M, int N, int K, int trans_b, int dtype, int fmt,
+                               int scales_mn_major, int num_cu, void* stream) {
+  if (int e = check_common(A, B, codes, sizes, G, N)) return e;
+  if (!scales) return set_error("null scale pointer");
+  if (M < 0 || K < 0) return set_error("negative M or K");
+  if (dtype != TGG_BF16 && dtype != TGG_F16) return set_error("data type code %d not supported", dtype);
+  if (fmt != DT_E4M3 && fmt != DT_E5M2) return set_error("unsupported fp8 format code %d", fmt);
+  if ((K & 7) || (N & 127)) return set_error("K must be a multiple of 8 and N of 128, got N=%d K=%d", N, K);
+  if (M == 0) return 0;
+  GemmParams p = zero_params();
+  p.A = A; p.B = B; p.C = codes; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
+  p.mode = MODE_MG; p.m_total = M; p.N = N; p.K = K;
+  p.a_sm = K; p.a_sk = 1;
+  p.b_sg = (int64_t)N * K;
+  if (trans_b) { p.b_sn = K; p.b_sk = 1; } else { p.b_sn = 1; p.b_sk = N; }
+  p.grid_limit = num_cu;
+  p.q_scales = scales;
+  p.q_fmt = fmt;
+  if (scales_mn_major) { p.q_rs = 1; p.q_bs = M; } else { p.q_rs = N / 128; p.q_bs = 1; }
+  const int layout = trans_b ? 0 : 1;
+  if (!fast_quant_supported(p, dtype, layout))
+    return set_error("shape outside the fused kernel's domain (G <= 512, K * 512 and N * 128 below 2^30 bytes): "
+                     "run tgg_m_grouped_gemm followed by tgg_per_token_cast_to_fp8, which gives the same bits");
+  return launch_fast_16bit_quant(p, dtype, layout, (hipStream_t)stream);
 }
 
 int tgg_m_grouped_gemm_padded(const void* A, const void* B, void* C, const void* sizes, int sizes_i64, int G,

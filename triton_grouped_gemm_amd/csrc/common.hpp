@@ -87,6 +87,11 @@ struct GemmParams {
   int tile_split;         // tuned kernels: 1 = per-XCD contiguous tile ranges (see sched_walk)
   int n_chunk;            // column tiles per chunk of the tile order, 0 = automatic (see sched_tile)
   int store_nt;           // tuned kernels: 1 = non-temporal output stores
+  // fused 1x128 quantisation of the output (tuned 16-bit M-grouped kernels): C then holds fp8 codes [rows, N] and
+  // the scale of (row, 128-column block) goes to q_scales[row * q_rs + block * q_bs]
+  float* q_scales;
+  int64_t q_rs, q_bs;
+  int q_fmt;              // DT_E4M3 / DT_E5M2; 0 = no quantisation
 };
 
 }  // namespace tgg

@@ -48,6 +48,16 @@ template <> struct Mma16<DT_F16> {
   }
 };
 
+// fp32 -> nearest 16-bit value of the output type (as fp32), and 16 bits -> fp32
+template <int DT> TGG_DEV float round16(float x) {
+  if (DT == DT_BF16) return (float)(__bf16)x;
+  return (float)(_Float16)x;
+}
+template <int DT> TGG_DEV float from16(uint16_t h) {
+  if (DT == DT_BF16) return __builtin_bit_cast(float, (uint32_t)h << 16);
+  return (float)__builtin_bit_cast(_Float16, h);
+}
+
 // Output store; nt = streaming hint (the output is written once and not read again by this kernel).
 TGG_DEV void store_c(i32x4_t* dst, i32x4_t v, int nt) {
   if (nt) __builtin_nontemporal_store(v, dst);
@@ -67,13 +77,14 @@ struct FastCfg {
   static constexpr int EPI_WAVE_BYTES = 32 * EPI_PITCH;
   static constexpr int SCHED_OFF = 2 * STAGE_BYTES;
   static constexpr int EPI_OFF = SCHED_OFF + (((int)sizeof(SchedTableT<kFastMaxGroups>) + 255) & ~255);
-  static constexpr int SMEM_BYTES = EPI_OFF + NWAVES * EPI_WAVE_BYTES;
+  static constexpr int QMAX_OFF = EPI_OFF + NWAVES * EPI_WAVE_BYTES;  // fused quantisation: [WN][BM] 16-bit row maxima
+  static constexpr int SMEM_BYTES = QMAX_OFF + WN * BM * 2;
   static_assert(NI_A % NWAVES == 0 && NI_B % NWAVES == 0, "copies must divide evenly over waves");
   static_assert(NWAVES % 4 == 0, "a wave keeps one swizzle pattern for all its copies");
   static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
 };
 
-template <class C, int DT, int LAYOUT>
+template <class C, int DT, int LAYOUT, bool QUANT>
 __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams p) {
   constexpr bool A_KMAJOR = LAYOUT != LAYOUT_TN;
   constexpr bool B_KMAJOR = LAYOUT == LAYOUT_NT;
@@ -356,6 +367,71 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
     const int64_t c_row0 = (LAYOUT == LAYOUT_TN) ? ((int64_t)cur.g * p.m_total + cur.row0) : cur.row0;
     char* const c_tile = (char*)p.C + ((c_row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2;
     const int st_row = lane >> 2, st_chunk = lane & 3;
+    if (QUANT) {
+      // Fused 1x128 quantisation, bit-identical to rounding the tile to the 16-bit type and quantising that:
+      // round, take each row's |max| over the wave's columns (own 32 values, then the partner lane's), exchange
+      // with the neighbouring wave that holds the other half of the 128-column block, scale, convert, store codes
+      // and one scale per (row, block).  A 128-column block never straddles tiles (N and the tile width are
+      // multiples of 128), and the maxima are exact 16-bit values, so they travel as 16 bits.
+      static_assert(!QUANT || (C::BN / C::WN == 64 && C::WN % 2 == 0), "two waves per 128-column block");
+      uint16_t* const rowmax = (uint16_t*)(smem + C::QMAX_OFF);
+      const int wn = wave % C::WN;
+      const float fmax_ = p.q_fmt == DT_E4M3 ? 448.0f : 57344.0f;
+      float rmax[C::TM];
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i) {
+        float m = 0.f;
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const float v = round16<DT>(acc[i][j][e]);
+            acc[i][j][e] = v;
+            m = fmaxf(m, fabsf(v));
+          }
+        m = fmaxf(m, __shfl_xor(m, 32, 64));
+        rmax[i] = m;
+        if (lh == 0) rowmax[wn * C::BM + wm0 + 32 * i + l32] = Out16<DT>::cvt(m);
+      }
+      __syncthreads();
+      char* const q_tile = (char*)p.C + (c_row0 + wm0) * (int64_t)p.N + cur.n0 + wn0;  // 1-byte codes
+      const int blk = (cur.n0 + wn0) >> 7;
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i) {
+        const float other = from16<DT>(rowmax[(wn ^ 1) * C::BM + wm0 + 32 * i + l32]);
+        const float amax = fmaxf(fmaxf(rmax[i], other), 1e-4f);
+        const float mult = (1.0f / amax) * fmax_;  // torch evaluates `448.0 / amax` as reciprocal * 448
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float a0 = acc[i][j][4 * q] * mult, a1 = acc[i][j][4 * q + 1] * mult;
+            const float a2 = acc[i][j][4 * q + 2] * mult, a3 = acc[i][j][4 * q + 3] * mult;
+            uint32_t w;
+            if (p.q_fmt == DT_E4M3) {
+              w = __builtin_amdgcn_cvt_pk_fp8_f32(a0, a1, 0u, false);
+              w = __builtin_amdgcn_cvt_pk_fp8_f32(a2, a3, w, true);
+            } else {
+              w = __builtin_amdgcn_cvt_pk_bf8_f32(a0, a1, 0u, false);
+              w = __builtin_amdgcn_cvt_pk_bf8_f32(a2, a3, w, true);
+            }
+            *(uint32_t*)(stage_c + l32 * C::EPI_PITCH + 32 * j + 8 * q + 4 * lh) = w;
+          }
+        // 32 rows x 64 one-byte codes are staged: 4 chunks of 16 bytes per row
+        const bool col_ok = cur.n0 + wn0 + st_chunk * 16 < p.N;
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+          const int r = it * 16 + st_row;
+          const i32x4_t v = *(const i32x4_t*)(stage_c + r * C::EPI_PITCH + st_chunk * 16);
+          if (col_ok && wm0 + 32 * i + r < cur.rows)
+            store_c((i32x4_t*)(q_tile + (int64_t)(32 * i + r) * p.N + st_chunk * 16), v, p.store_nt);
+        }
+        const int row = wm0 + 32 * i + l32;
+        if ((wn & 1) == 0 && lh == 0 && row < cur.rows && cur.n0 + wn0 < p.N)
+          p.q_scales[(c_row0 + row) * p.q_rs + (int64_t)blk * p.q_bs] = amax / fmax_;
+      }
+      continue;
+    }
 #pragma unroll
     for (int i = 0; i < C::TM; ++i) {
 #pragma unroll
@@ -378,12 +454,12 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   wait_vmcnt<0>();  // the trailing zero-length copies still write LDS: let them finish before the wave ends
 }
 
-template <class C, int DT, int LAYOUT>
+template <class C, int DT, int LAYOUT, bool QUANT>
 int launch_cfg(const GemmParams& p, hipStream_t s) {
   static bool attr_set[64] = {false};
   int dev = 0;
   (void)hipGetDevice(&dev);
-  auto kern = gemm_fast_kernel<C, DT, LAYOUT>;
+  auto kern = gemm_fast_kernel<C, DT, LAYOUT, QUANT>;
   if (dev >= 0 && dev < 64 && !attr_set[dev]) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM_BYTES) != hipSuccess)
       return check_launch("hipFuncSetAttribute(gemm_fast)");
@@ -401,8 +477,8 @@ template <int DT, int LAYOUT>
 int launch_variant(const GemmParams& p, hipStream_t s) {
   switch (g_variant) {
     default:
-    case 0: return launch_cfg<FastCfg<256, 256, 2, 4>, DT, LAYOUT>(p, s);
-    case 1: return launch_cfg<FastCfg<256, 128, 2, 4>, DT, LAYOUT>(p, s);
+    case 0: return launch_cfg<FastCfg<256, 256, 2, 4>, DT, LAYOUT, false>(p, s);
+    case 1: return launch_cfg<FastCfg<256, 128, 2, 4>, DT, LAYOUT, false>(p, s);
   }
 }
 
@@ -432,6 +508,21 @@ bool fast_supported(const GemmParams& p, int dt, int layout) {
   if ((int64_t)p.K * 2 * 256 >= (1ll << 30)) return false;
   if (layout == LAYOUT_NN && (int64_t)p.N * 2 * 64 >= (1ll << 30)) return false;
   return layout == LAYOUT_NT || layout == LAYOUT_NN;
+}
+
+// Fused-quantisation launches: M-grouped NT / NN with N a multiple of 128 (see fast_quant_supported).
+int launch_fast_16bit_quant(const GemmParams& p, int dt, int layout, hipStream_t s) {
+  typedef FastCfg<256, 256, 2, 4> Cfg;
+  if (dt == DT_BF16)
+    return layout == LAYOUT_NT ? launch_cfg<Cfg, DT_BF16, LAYOUT_NT, true>(p, s) : launch_cfg<Cfg, DT_BF16, LAYOUT_NN, true>(p, s);
+  return layout == LAYOUT_NT ? launch_cfg<Cfg, DT_F16, LAYOUT_NT, true>(p, s) : launch_cfg<Cfg, DT_F16, LAYOUT_NN, true>(p, s);
+}
+
+bool fast_quant_supported(const GemmParams& p, int dt, int layout) {
+  if (layout != LAYOUT_NT && layout != LAYOUT_NN) return false;
+  if (p.mode != MODE_MG && p.mode != MODE_MG_PAD) return false;
+  if ((p.N & 127) != 0) return false;
+  return fast_supported(p, dt, layout);
 }
 
 int launch_fast_16bit(const GemmParams& p, int dt, int layout, hipStream_t s) {
