@@ -59,21 +59,23 @@ constexpr int kSlabRowBytes = 128;  // a slab holds 128 bytes of every K-contigu
 //   KMAJOR: ROWS rows of 128 bytes (64 K values each).  A copy instruction covers 8 rows; the
 //           16-byte chunk c of row r sits at slot c ^ ((r / 2) % 8).
 //   !KMAJOR: 64 token rows of ROWS*2 bytes.  A copy instruction covers 1024 / (ROWS*2) token rows;
-//           chunk c of token row k sits at slot c ^ ((k % 4) * 4).
+//           chunk c of token row k sits at slot c ^ ((k % 4) * 4) ^ ((k / 8 % 2) * 2): the transposing fragment
+//           read of a wave touches token rows 8 g + e (g = 0..3, e = 0..3) at the same columns, and this spreads
+//           them over all banks.
 template <int ROWS, bool KMAJOR> struct Operand {
   static constexpr int SLAB_BYTES = ROWS * kSlabRowBytes;
   static constexpr int NI = SLAB_BYTES / 1024;                 // copy instructions per slab
   static constexpr int ROW_BYTES = KMAJOR ? kSlabRowBytes : ROWS * 2;  // bytes of one LDS row (token rows: 16-bit)
   static constexpr int CPR = ROW_BYTES / 16;                   // 16-byte chunks per LDS row
   static constexpr int RPI = 1024 / ROW_BYTES;                 // LDS rows per copy instruction
-  static constexpr int NPAT = KMAJOR ? 2 : (RPI >= 4 ? 1 : 4 / RPI);  // swizzle patterns over instructions
+  static constexpr int NPAT = KMAJOR ? 2 : (RPI >= 16 ? 1 : 16 / RPI);  // swizzle patterns over instructions
 
   // byte offset (from the slab's first byte in global memory) fetched by `lane` of a copy
   // instruction with swizzle pattern `pat`; ld = bytes between consecutive global rows.
   static TGG_DEV int lane_voff(int lane, int pat, int ld) {
     const int r_local = lane / CPR, slot = lane % CPR;
     const int r = pat * RPI + r_local;  // row index modulo the swizzle period
-    const int sw = KMAJOR ? (r / 2) % 8 : (r % 4) * 4;
+    const int sw = KMAJOR ? (r / 2) % 8 : ((r % 4) * 4) ^ ((r / 8 % 2) * 2);
     return r_local * ld + ((slot ^ sw) << 4);
   }
   // K-contiguous rows only: which 16-byte chunk of its row (0..7) that lane fetches

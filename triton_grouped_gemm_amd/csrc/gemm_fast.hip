@@ -22,10 +22,14 @@
 //   * K-contiguous operands are read back as 16-byte MFMA fragments (ds_read_b128); operands whose
 //     rows are tokens (MN-contiguous) are read with the transposing ds_read_b64_tr_b16, which hands
 //     every lane 4 consecutive K values of one column.
-//   * Each wave owns a (BM/WM) x (BN/WN) block of 32x32x16 MFMA tiles, issued with the B operand as
-//     srcA and the A operand as srcB, so a lane ends up with 4 consecutive output columns of one
-//     row; results are transposed 32x32 block by block through a small per-wave LDS staging area
-//     (separate from the slab buffers, so the copy stream keeps running) and leave as 16-byte stores.
+//   * Each wave owns a (BM/WM) x (BN/WN) block of 16x16x32 MFMA tiles.  That shape is chosen for power: with
+//     all 256 CUs multiplying random operands the chip is power-limited, and 16x16x32 delivers about 20 % more
+//     flops per watt than 32x32x16 (a quarter of the accumulator traffic per multiply-add pair of operands);
+//     it also keeps full issue rate with two waves per SIMD, which 32x32x16 with distinct operand registers
+//     does not.  Multiplies are issued with the B operand as srcA and the A operand as srcB, so a lane ends up
+//     with 4 consecutive output columns of one row; results are transposed one 16-row strip at a time through a
+//     small per-wave LDS staging area (separate from the slab buffers, so the copy stream keeps running) and
+//     leave as 16-byte stores that cover whole row segments of the wave's columns.
 #include "fast_common.hpp"
 #include "launch.hpp"
 
@@ -38,13 +42,13 @@ constexpr int BK = 64;  // K depth of a slab for 16-bit operands
 
 template <int DT> struct Mma16;
 template <> struct Mma16<DT_BF16> {
-  static TGG_DEV f32x16_t run(i32x4_t w, i32x4_t x, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, w), __builtin_bit_cast(bf16x8_t, x), c, 0, 0, 0);
+  static TGG_DEV f32x4_t run(i32x4_t w, i32x4_t x, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, w), __builtin_bit_cast(bf16x8_t, x), c, 0, 0, 0);
   }
 };
 template <> struct Mma16<DT_F16> {
-  static TGG_DEV f32x16_t run(i32x4_t w, i32x4_t x, f32x16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, w), __builtin_bit_cast(f16x8_t, x), c, 0, 0, 0);
+  static TGG_DEV f32x4_t run(i32x4_t w, i32x4_t x, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, w), __builtin_bit_cast(f16x8_t, x), c, 0, 0, 0);
   }
 };
 
@@ -72,15 +76,15 @@ struct FastCfg {
   static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   static constexpr int NI_A = A_BYTES / 1024, NI_B = B_BYTES / 1024;
-  static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-  static constexpr int EPI_PITCH = 32 * 2 + 16;  // staged 32x32 output block: row pitch in bytes
-  static constexpr int EPI_WAVE_BYTES = 32 * EPI_PITCH;
+  static constexpr int TM = BM / WM / 16, TN = BN / WN / 16;  // 16x16 blocks per wave
+  static constexpr int EPI_PITCH = TN * 32 + 16;  // staged strip of 16 rows x (16 TN) 16-bit outputs: row pitch in bytes
+  static constexpr int EPI_WAVE_BYTES = 16 * EPI_PITCH;
   static constexpr int SCHED_OFF = 2 * STAGE_BYTES;
   static constexpr int EPI_OFF = SCHED_OFF + (((int)sizeof(SchedTableT<kFastMaxGroups>) + 255) & ~255);
   static constexpr int QMAX_OFF = EPI_OFF + NWAVES * EPI_WAVE_BYTES;  // fused quantisation: [WN][BM] 16-bit row maxima
   static constexpr int SMEM_BYTES = QMAX_OFF + WN * BM * 2;
   static_assert(NI_A % NWAVES == 0 && NI_B % NWAVES == 0, "copies must divide evenly over waves");
-  static_assert(NWAVES % 4 == 0, "a wave keeps one swizzle pattern for all its copies");
+  static_assert(NWAVES % 8 == 0, "a wave keeps one swizzle pattern for all its copies");
   static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
 };
 
@@ -101,7 +105,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm0 = (wave / C::WN) * (C::BM / C::WM);
   const int wn0 = (wave % C::WN) * (C::BN / C::WN);
-  const int l32 = lane & 31, lh = lane >> 5;
+  const int l16 = lane & 15, lg = lane >> 4;
 
   // global row pitches in bytes
   const int64_t a_ld = (LAYOUT == LAYOUT_TN ? p.m_total : (int64_t)p.K) * 2;
@@ -116,59 +120,51 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   const int a_voff_tail = (A_KMAJOR && OpA::lane_chunk(lane, wave % OpA::NPAT) >= tail_chunks) ? kNoFetch : a_voff;
   const int b_voff_tail = (B_KMAJOR && OpB::lane_chunk(lane, wave % OpB::NPAT) >= tail_chunks) ? kNoFetch : b_voff;
 
-  // per-lane LDS offsets of the fragment reads, relative to the operand's slab
-  //   K-contiguous: 16 bytes = K values 16 ks + 8 lh + (0..7) of row (block + l32)
-  //   token rows:   lane L of a 16-lane group loads 8 bytes of token row (L % 16) / 4; the transposing
-  //                 read returns to lane i the 4 tokens of column i of the group
-  int a_rd[A_KMAJOR ? BK / 16 : C::TM];
-  int b_rd[B_KMAJOR ? BK / 16 : C::TN];
+  // per-lane LDS offsets of the fragment reads, relative to the operand's slab.  A fragment of the 16x16x32
+  // multiply is 8 consecutive K values per lane: K = 32 ks + 8 lg + (0..7) of row or column (block + l16).
+  //   K-contiguous: one 16-byte read
+  //   token rows:   two transposing 8-byte reads (K 8 lg + 0..3 and + 4..7).  Lane L of a 16-lane group addresses
+  //                 8 bytes (4 columns) of token row L / 4; the read returns to lane i the 4 tokens of column i.
+  constexpr int KSTEPS = BK / 32;
+  int a_rd[A_KMAJOR ? KSTEPS : C::TM];
+  int b_rd[B_KMAJOR ? KSTEPS : C::TN];
   if (A_KMAJOR) {
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) a_rd[ks] = (wm0 + l32) * 128 + (((2 * ks + lh) ^ ((l32 / 2) % 8)) << 4);
+    for (int ks = 0; ks < KSTEPS; ++ks) a_rd[ks] = (wm0 + l16) * 128 + (((4 * ks + lg) ^ ((l16 / 2) % 8)) << 4);
   } else {
 #pragma unroll
     for (int i = 0; i < C::TM; ++i) {
-      const int blk = lane >> 4, j = lane & 15, e = j >> 2, c = j & 3;
-      const int chunk = ((wm0 + 32 * i) / 8 + (blk & 1) * 2 + (c >> 1)) ^ (e * 4);
-      a_rd[i] = ((blk >> 1) * 8 + e) * (C::BM * 2) + chunk * 16 + (c & 1) * 8;
+      const int e = l16 >> 2, c = l16 & 3;
+      const int chunk = ((wm0 + 16 * i) / 8 + (c >> 1)) ^ (e * 4) ^ ((lg & 1) * 2);
+      a_rd[i] = (lg * 8 + e) * (C::BM * 2) + chunk * 16 + (c & 1) * 8;
     }
   }
   if (B_KMAJOR) {
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) b_rd[ks] = (wn0 + l32) * 128 + (((2 * ks + lh) ^ ((l32 / 2) % 8)) << 4);
+    for (int ks = 0; ks < KSTEPS; ++ks) b_rd[ks] = (wn0 + l16) * 128 + (((4 * ks + lg) ^ ((l16 / 2) % 8)) << 4);
   } else {
 #pragma unroll
     for (int j2 = 0; j2 < C::TN; ++j2) {
-      const int blk = lane >> 4, j = lane & 15, e = j >> 2, c = j & 3;
-      const int chunk = ((wn0 + 32 * j2) / 8 + (blk & 1) * 2 + (c >> 1)) ^ (e * 4);
-      b_rd[j2] = ((blk >> 1) * 8 + e) * (C::BN * 2) + chunk * 16 + (c & 1) * 8;
+      const int e = l16 >> 2, c = l16 & 3;
+      const int chunk = ((wn0 + 16 * j2) / 8 + (c >> 1)) ^ (e * 4) ^ ((lg & 1) * 2);
+      b_rd[j2] = (lg * 8 + e) * (C::BN * 2) + chunk * 16 + (c & 1) * 8;
     }
   }
-  // MFMA fragments of K step ks of the slab at sa (A part) / sb (B part)
-  auto load_frags = [&](const char* sa, int ks, i32x4_t (&fa)[C::TM], i32x4_t (&fb)[C::TN]) {
-    const char* sb = sa + C::A_BYTES;
-#pragma unroll
-    for (int i = 0; i < C::TM; ++i) {
-      if (A_KMAJOR) {
-        fa[i] = *(const i32x4_t*)(sa + a_rd[ks] + i * 32 * 128);
-      } else {
-        const char* q = sa + a_rd[i] + ks * 16 * (C::BM * 2);
-        const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)q);
-        const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)(q + 4 * (C::BM * 2)));
-        fa[i] = __builtin_bit_cast(i32x4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < C::TN; ++j) {
-      if (B_KMAJOR) {
-        fb[j] = *(const i32x4_t*)(sb + b_rd[ks] + j * 32 * 128);
-      } else {
-        const char* q = sb + b_rd[j] + ks * 16 * (C::BN * 2);
-        const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)q);
-        const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)(q + 4 * (C::BN * 2)));
-        fb[j] = __builtin_bit_cast(i32x4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-      }
-    }
+  // MFMA fragment of K step ks: block i of A / block j of B of the slab at s
+  auto load_a = [&](const char* s, int ks, int i) -> i32x4_t {
+    if (A_KMAJOR) return *(const i32x4_t*)(s + a_rd[ks] + i * 16 * 128);
+    const char* q = s + a_rd[i] + ks * 32 * (C::BM * 2);
+    const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)q);
+    const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)(q + 4 * (C::BM * 2)));
+    return __builtin_bit_cast(i32x4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+  auto load_b = [&](const char* s, int ks, int j) -> i32x4_t {
+    const char* sb = s + C::A_BYTES;
+    if (B_KMAJOR) return *(const i32x4_t*)(sb + b_rd[ks] + j * 16 * 128);
+    const char* q = sb + b_rd[j] + ks * 32 * (C::BN * 2);
+    const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)q);
+    const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)(q + 4 * (C::BN * 2)));
+    return __builtin_bit_cast(i32x4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
   // Slab sequence of a tile, held in scalar registers: where the next slab of each operand starts and how far
@@ -254,8 +250,8 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
     bool tail;  // the tile's last slab, cut short by K
   };
   constexpr int CA = C::NI_A / C::NWAVES, CB = C::NI_B / C::NWAVES, NC = CA + CB;
-  constexpr int SP = (C::TM * C::TN) / (NC / 2);  // multiplies between two copies
-  static_assert(NC % 2 == 0 && SP >= 1, "a slab's copies are spread over the multiplies of two K steps");
+  constexpr int SP = (C::TM * C::TN / 2) / (NC / 2);  // multiplies between two copies
+  static_assert(NC % 2 == 0 && SP >= 1, "a slab's copies are spread over the multiplies of two half K steps");
   auto begin_slab = [&](int buf) {
     SlabCopy sc;
     const bool live = feed.issued < feed.kt_n;
@@ -283,18 +279,20 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
     }
   };
 
-  // Epilogue staging: a private 32x32 block of 16-bit outputs per wave, rows padded by 16 bytes.
-  char* const stage_c = smem + C::EPI_OFF + wave * C::EPI_WAVE_BYTES;
-
-  // Software pipeline.  Per slab r (4 K steps of 16):
-  //   steps 0..2  read the fragments of the following step while multiplying the current one;
-  //   step 3      wait for this wave's share of slab r+1, workgroup barrier (now slab r+1 is complete and
-  //               nobody reads slab r any more: its last fragments are already in registers), read step 0
-  //               of slab r+1, and only then multiply step 3.
-  // The copies of slab r+2 (into slab r's buffer) are issued one per two multiplies during step 3 and
-  // the following step 0: the texture-address unit takes 16 cycles per copy instruction and its queue
-  // is short, so a wave that issues its copies back to back sits blocked behind the other waves'
-  // copies with its multiplies queued up behind them.  Tile boundaries do not interrupt the stream.
+  // Software pipeline.  A slab is two K steps of 32, each issued as two halves (row blocks 0..TM/2-1, then the
+  // rest).  Registers hold one K step of A fragments (replaced one by one: as soon as the multiplies of row
+  // block i are issued, fragment i of the following step is read into its place; the last block alternates
+  // between two registers so that its successor can be read early) and two K steps of B fragments.  Per slab r:
+  //   step 0            multiply while reading step 1 of the same slab;
+  //   step 1, 1st half  multiply only;
+  //   then wait for this wave's share of slab r+1 and pass the workgroup barrier: slab r+1 is complete and
+  //   nobody reads slab r any more, its last fragments are already in registers;
+  //   step 1, 2nd half  multiply while reading step 0 of slab r+1 (first the fragments the 1st half skipped).
+  // The copies of slab r+2 (into slab r's buffer) are issued one per SP multiplies during the half step after
+  // the barrier and the half step after that, which leaves them a whole K step to land before they are waited
+  // for.  They are spread out because the texture-address unit takes 16 cycles per copy instruction and its
+  // queue is short: a wave that issues its copies back to back sits blocked behind the other waves' copies with
+  // its multiplies queued up behind them.  Tile boundaries do not interrupt the stream.
   feed_seek(walk.first);
   {
     const SlabCopy s0 = begin_slab(0);
@@ -306,36 +304,55 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   SlabCopy sc = begin_slab(1);
 #pragma unroll
   for (int k = 0; k < NC / 2; ++k) copy_k(sc, k);
-  i32x4_t fa0[C::TM], fb0[C::TN], fa1[C::TM], fb1[C::TN];
-  load_frags(smem, 0, fa0, fb0);
+  i32x4_t fa[C::TM - 1], fa_last[2], fb[2][C::TN];
+#pragma unroll
+  for (int i = 0; i < C::TM - 1; ++i) fa[i] = load_a(smem, 0, i);
+  fa_last[0] = load_a(smem, 0, C::TM - 1);
+#pragma unroll
+  for (int j = 0; j < C::TN; ++j) fb[0][j] = load_b(smem, 0, j);
   int ring = 0;
 
   for (int64_t tile_id = walk.first; tile_id < walk.end; tile_id += walk.stride) {
     const Tile cur = sched_tile<C::BM, C::BN>(p, sched, tile_id);
     const int kt_n = __builtin_amdgcn_readfirstlane(slabs_of(cur));
-    f32x16_t acc[C::TM][C::TN];
+    f32x4_t acc[C::TM][C::TN];
 #pragma unroll
     for (int i = 0; i < C::TM; ++i)
 #pragma unroll
       for (int j = 0; j < C::TN; ++j)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
 
-    // One K step: multiply (fa, fb); right after the first multiply, read the fragments of K step ks_next
-    // of the slab at s_next into (fna, fnb); copies [k0, k0 + NC/2) of `sc` are issued one per SP
-    // multiplies when k0 >= 0.
+    // Half a K step: the multiplies of row blocks [h TM/2, (h+1) TM/2) with fragment set `cur_set`.  Meanwhile
+    // fragments of K step ks_next of the slab at s_next are read into the other set:
+    //   READ_EARLY    B fragments and the last A fragment right after the first multiply, A fragment i after the
+    //                 multiplies of row block i;
+    //   READ_ROLL     A fragment i after the multiplies of row block i;
+    //   READ_NONE     nothing (the slab to read from is not complete yet);
+    //   READ_CATCH_UP as READ_EARLY, plus the A fragments that the preceding READ_NONE half left out.
+    // Copies [k0, k0 + NC/2) of `sc` are issued one per SP multiplies when k0 >= 0.
+    enum { READ_EARLY, READ_ROLL, READ_NONE, READ_CATCH_UP };
     SlabCopy sc_next;
-    auto step = [&](const i32x4_t (&fa)[C::TM], const i32x4_t (&fb)[C::TN], const char* s_next, int ks_next,
-                    i32x4_t (&fna)[C::TM], i32x4_t (&fnb)[C::TN], int k0, bool prepare = false) {
+    auto half = [&](int cur_set, int h, const char* s_next, int ks_next, int mode, int k0, bool prepare = false) {
+      const int nxt = cur_set ^ 1;
+      constexpr int HM = C::TM / 2;
 #pragma unroll
-      for (int i = 0; i < C::TM; ++i)
+      for (int ii = 0; ii < HM; ++ii) {
+        const int i = h * HM + ii;
+        const i32x4_t a = i == C::TM - 1 ? fa_last[cur_set] : fa[i];
 #pragma unroll
         for (int j = 0; j < C::TN; ++j) {
-          acc[i][j] = Mma16<DT>::run(fb[j], fa[i], acc[i][j]);
-          const int n = i * C::TN + j;
-          if (n == 0) {
+          acc[i][j] = Mma16<DT>::run(fb[cur_set][j], a, acc[i][j]);
+          const int n = ii * C::TN + j;
+          if (n == 0 && (mode == READ_EARLY || mode == READ_CATCH_UP)) {
             __builtin_amdgcn_sched_barrier(0);
-            load_frags(s_next, ks_next, fna, fnb);
+#pragma unroll
+            for (int j2 = 0; j2 < C::TN; ++j2) fb[nxt][j2] = load_b(s_next, ks_next, j2);
+            fa_last[nxt] = load_a(s_next, ks_next, C::TM - 1);
+            if (mode == READ_CATCH_UP) {
+#pragma unroll
+              for (int i2 = 0; i2 < HM; ++i2) fa[i2] = load_a(s_next, ks_next, i2);
+            }
             __builtin_amdgcn_sched_barrier(0);
           }
           if (prepare && n == 1) sc_next = begin_slab(ring & 1);  // scalar work, under the multiplies just issued
@@ -345,34 +362,45 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
             __builtin_amdgcn_sched_barrier(0);
           }
         }
+        if (mode != READ_NONE && i < C::TM - 1) {
+          __builtin_amdgcn_sched_barrier(0);
+          fa[i] = load_a(s_next, ks_next, i);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
     };
 
     for (int kt = 0; kt < kt_n; ++kt) {
       const char* sa = smem + (ring & 1) * C::STAGE_BYTES;
       const char* sn = smem + ((ring + 1) & 1) * C::STAGE_BYTES;
-      step(fa0, fb0, sa, 1, fa1, fb1, NC / 2);
-      step(fa1, fb1, sa, 2, fa0, fb0, -1);
-      step(fa0, fb0, sa, 3, fa1, fb1, -1, true);
+      half(0, 0, sa, 1, READ_EARLY, NC / 2);
+      half(0, 1, sa, 1, READ_ROLL, -1, true);
+      half(1, 0, sn, 0, READ_NONE, -1);
       wait_vmcnt<0>();
       __syncthreads();
       sc = sc_next;
-      step(fa1, fb1, sn, 0, fa0, fb0, 0);
+      half(1, 1, sn, 0, READ_CATCH_UP, 0);
       ++ring;
     }
 
-    // Epilogue.  A lane owns row l32 and columns 32 j + 8 q + 4 lh + (0..3) of each 32-row block i:
-    // transpose each 32x32 block through the wave's LDS staging so that global stores are 16 bytes per
-    // lane and 64-byte row segments, two neighbouring rows' worth per 128 bytes of a wave's store.
+    // Epilogue.  A lane owns row l16 and columns 16 j + 4 lg + (0..3) of each 16-row block i: transpose one
+    // 16-row strip (all of the wave's columns) at a time through the wave's LDS staging so that global stores
+    // are 16 bytes per lane and cover whole row segments.  The lane id passes through an opaque statement so
+    // that the address arithmetic below is redone per tile instead of being hoisted out of the tile loop, where
+    // it would occupy registers (or spill) across the multiplies.
+    int el = lane;
+    asm volatile("" : "+v"(el));
+    const int e16 = el & 15, eg = el >> 4;
+    char* const stage_c = smem + C::EPI_OFF + wave * C::EPI_WAVE_BYTES;
     const int64_t c_row0 = (LAYOUT == LAYOUT_TN) ? ((int64_t)cur.g * p.m_total + cur.row0) : cur.row0;
-    char* const c_tile = (char*)p.C + ((c_row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2;
-    const int st_row = lane >> 2, st_chunk = lane & 3;
     if (QUANT) {
       // Fused 1x128 quantisation, bit-identical to rounding the tile to the 16-bit type and quantising that:
-      // round, take each row's |max| over the wave's columns (own 32 values, then the partner lane's), exchange
-      // with the neighbouring wave that holds the other half of the 128-column block, scale, convert, store codes
-      // and one scale per (row, block).  A 128-column block never straddles tiles (N and the tile width are
-      // multiples of 128), and the maxima are exact 16-bit values, so they travel as 16 bits.
+      // round, take each row's |max| over the wave's columns (own 16 values, then the three lanes that hold the
+      // rest of the row), exchange with the neighbouring wave that holds the other half of the 128-column block,
+      // scale, convert, store codes and one scale per (row, block).  A 128-column block never straddles tiles
+      // (N and the tile width are multiples of 128), and the maxima are exact 16-bit values, so they travel as
+      // 16 bits.
       static_assert(!QUANT || (C::BN / C::WN == 64 && C::WN % 2 == 0), "two waves per 128-column block");
       uint16_t* const rowmax = (uint16_t*)(smem + C::QMAX_OFF);
       const int wn = wave % C::WN;
@@ -384,70 +412,65 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
 #pragma unroll
         for (int j = 0; j < C::TN; ++j)
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
+          for (int e = 0; e < 4; ++e) {
             const float v = round16<DT>(acc[i][j][e]);
             acc[i][j][e] = v;
             m = fmaxf(m, fabsf(v));
           }
+        m = fmaxf(m, __shfl_xor(m, 16, 64));
         m = fmaxf(m, __shfl_xor(m, 32, 64));
         rmax[i] = m;
-        if (lh == 0) rowmax[wn * C::BM + wm0 + 32 * i + l32] = Out16<DT>::cvt(m);
+        if (eg == 0) rowmax[wn * C::BM + wm0 + 16 * i + e16] = Out16<DT>::cvt(m);
       }
       __syncthreads();
       char* const q_tile = (char*)p.C + (c_row0 + wm0) * (int64_t)p.N + cur.n0 + wn0;  // 1-byte codes
       const int blk = (cur.n0 + wn0) >> 7;
+      const int st_row = el >> 2, st_chunk = el & 3;  // 16 rows x 64 one-byte codes are staged: 4 chunks of 16 bytes per row
+      const bool col_ok = cur.n0 + wn0 + st_chunk * 16 < p.N;
 #pragma unroll
       for (int i = 0; i < C::TM; ++i) {
-        const float other = from16<DT>(rowmax[(wn ^ 1) * C::BM + wm0 + 32 * i + l32]);
+        const float other = from16<DT>(rowmax[(wn ^ 1) * C::BM + wm0 + 16 * i + e16]);
         const float amax = fmaxf(fmaxf(rmax[i], other), 1e-4f);
         const float mult = (1.0f / amax) * fmax_;  // torch evaluates `448.0 / amax` as reciprocal * 448
 #pragma unroll
-        for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const float a0 = acc[i][j][4 * q] * mult, a1 = acc[i][j][4 * q + 1] * mult;
-            const float a2 = acc[i][j][4 * q + 2] * mult, a3 = acc[i][j][4 * q + 3] * mult;
-            uint32_t w;
-            if (p.q_fmt == DT_E4M3) {
-              w = __builtin_amdgcn_cvt_pk_fp8_f32(a0, a1, 0u, false);
-              w = __builtin_amdgcn_cvt_pk_fp8_f32(a2, a3, w, true);
-            } else {
-              w = __builtin_amdgcn_cvt_pk_bf8_f32(a0, a1, 0u, false);
-              w = __builtin_amdgcn_cvt_pk_bf8_f32(a2, a3, w, true);
-            }
-            *(uint32_t*)(stage_c + l32 * C::EPI_PITCH + 32 * j + 8 * q + 4 * lh) = w;
+        for (int j = 0; j < C::TN; ++j) {
+          const float a0 = acc[i][j][0] * mult, a1 = acc[i][j][1] * mult;
+          const float a2 = acc[i][j][2] * mult, a3 = acc[i][j][3] * mult;
+          uint32_t w;
+          if (p.q_fmt == DT_E4M3) {
+            w = __builtin_amdgcn_cvt_pk_fp8_f32(a0, a1, 0u, false);
+            w = __builtin_amdgcn_cvt_pk_fp8_f32(a2, a3, w, true);
+          } else {
+            w = __builtin_amdgcn_cvt_pk_bf8_f32(a0, a1, 0u, false);
+            w = __builtin_amdgcn_cvt_pk_bf8_f32(a2, a3, w, true);
           }
-        // 32 rows x 64 one-byte codes are staged: 4 chunks of 16 bytes per row
-        const bool col_ok = cur.n0 + wn0 + st_chunk * 16 < p.N;
-#pragma unroll
-        for (int it = 0; it < 2; ++it) {
-          const int r = it * 16 + st_row;
-          const i32x4_t v = *(const i32x4_t*)(stage_c + r * C::EPI_PITCH + st_chunk * 16);
-          if (col_ok && wm0 + 32 * i + r < cur.rows)
-            store_c((i32x4_t*)(q_tile + (int64_t)(32 * i + r) * p.N + st_chunk * 16), v, p.store_nt);
+          *(uint32_t*)(stage_c + e16 * C::EPI_PITCH + 16 * j + 4 * eg) = w;
         }
-        const int row = wm0 + 32 * i + l32;
-        if ((wn & 1) == 0 && lh == 0 && row < cur.rows && cur.n0 + wn0 < p.N)
+        const i32x4_t v = *(const i32x4_t*)(stage_c + st_row * C::EPI_PITCH + st_chunk * 16);
+        if (col_ok && wm0 + 16 * i + st_row < cur.rows)
+          store_c((i32x4_t*)(q_tile + (int64_t)(16 * i + st_row) * p.N + st_chunk * 16), v, p.store_nt);
+        const int row = wm0 + 16 * i + e16;
+        if ((wn & 1) == 0 && eg == 0 && row < cur.rows && cur.n0 + wn0 < p.N)
           p.q_scales[(c_row0 + row) * p.q_rs + (int64_t)blk * p.q_bs] = amax / fmax_;
       }
       continue;
     }
+    char* const c_tile = (char*)p.C + ((c_row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2;
+    constexpr int CPS = 2 * C::TN;        // 16-byte chunks per staged row
+    constexpr int PASSES = 16 * CPS / 64;  // wave-wide reads per strip
+    static_assert(16 * CPS % 64 == 0, "a strip is read back by whole waves");
 #pragma unroll
     for (int i = 0; i < C::TM; ++i) {
 #pragma unroll
-      for (int j = 0; j < C::TN; ++j) {
+      for (int j = 0; j < C::TN; ++j)
+        *(uint2*)(stage_c + e16 * C::EPI_PITCH + (16 * j + 4 * eg) * 2) =
+            pack4<DT>(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          *(uint2*)(stage_c + l32 * C::EPI_PITCH + (8 * q + 4 * lh) * 2) =
-              pack4<DT>(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
-        const bool col_ok = cur.n0 + wn0 + 32 * j + st_chunk * 8 < p.N;
-#pragma unroll
-        for (int it = 0; it < 2; ++it) {
-          const int r = it * 16 + st_row;
-          const i32x4_t v = *(const i32x4_t*)(stage_c + r * C::EPI_PITCH + st_chunk * 16);
-          if (col_ok && wm0 + 32 * i + r < cur.rows)
-            store_c((i32x4_t*)(c_tile + ((int64_t)(32 * i + r) * p.N + 32 * j + st_chunk * 8) * 2), v, p.store_nt);
-        }
+      for (int it = 0; it < PASSES; ++it) {
+        const int idx = it * 64 + el, r = idx / CPS, ch = idx % CPS;
+        const i32x4_t v = *(const i32x4_t*)(stage_c + r * C::EPI_PITCH + ch * 16);
+        if (cur.n0 + wn0 + ch * 8 < p.N && wm0 + 16 * i + r < cur.rows)
+          store_c((i32x4_t*)(c_tile + ((int64_t)(16 * i + r) * p.N + ch * 8) * 2), v, p.store_nt);
       }
     }
   }
