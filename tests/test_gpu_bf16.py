@@ -126,6 +126,30 @@ def test_contiguous_padded_bf16(dev, variant):
         start += p
 
 
+@pytest.mark.parametrize("psum", [False, True])
+def test_contiguous_padded_bf16_explicit_layout(dev, psum):
+    # the explicit layout, not size_per_group, says which rows are valid: same padded placement, fewer valid rows
+    from triton_grouped_gemm_amd.gemm import layout as L
+    sizes = [100, 0, 128, 300]
+    in_layout = [90, 0, 128, 257]
+    padded = [128, 0, 128, 384]
+    Mp, N, K = sum(padded), 256, 128
+    a = _randn((Mp, K), K ** -0.5, 19)
+    b = _randn((4, N, K), 1.0, 20)
+    lay = (L.make_deep_gemm_psum_layout(in_layout) if psum else L.make_deep_gemm_grouped_layout(in_layout)).to(dev)
+    out = torch.full((Mp, N), 3.0, dtype=torch.bfloat16, device=dev)
+    m_grouped_bf16_nt_contiguous(a.to(dev), b.to(dev), torch.tensor(sizes, dtype=torch.int32, device=dev), out=out,
+                                 grouped_layout=lay, use_psum_layout=psum)
+    out = out.cpu()
+    start = 0
+    for g, (s, p) in enumerate(zip(in_layout, padded)):
+        if s:
+            check_16bit_gemm(out[start:start + s], a[start:start + s] @ b[g].t(),
+                             a[start:start + s].float() @ b[g].float().t(), f"layout g{g}")
+        assert torch.equal(out[start + s:start + p], torch.full((p - s, N), 3.0, dtype=torch.bfloat16))
+        start += p
+
+
 @pytest.mark.parametrize("trans_b", [True, False])
 def test_masked_small(dev, variant, trans_b):
     G, m_max, N, K = 6, 256, 264, 192

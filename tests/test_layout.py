@@ -75,3 +75,14 @@ def test_metadata_builder_matches_oracle():
     assert idx[: len(ridx)].tolist() == ridx and int(mpad) == rmpad
     assert idx.numel() == sum(sizes) // 128 + len(sizes) and idx.dtype == torch.int32
     assert ps.dtype == torch.int32 and gs.dtype == torch.int64
+
+
+def test_sizes_from_explicit_layouts():
+    # both explicit layout forms give back the valid rows they were built from (reference gemm/layout.py:73-119)
+    from triton_grouped_gemm_amd.gemm.deep_gemm_ops import sizes_from_layout
+    for sizes, block_m in ([[3, 5, 0, 7], 4], [[0, 0, 9], 8], [[128, 1, 127, 256, 0], 128], [[5], 128]):
+        rows = L.make_deep_gemm_grouped_layout(sizes, block_m=block_m)
+        ends = L.make_deep_gemm_psum_layout(sizes, block_m=block_m)
+        assert sizes_from_layout(rows, len(sizes), block_m, False).tolist() == sizes
+        assert sizes_from_layout(ends, len(sizes), block_m, True).tolist() == sizes
+        assert sizes_from_layout(rows.to(torch.int64), len(sizes), block_m, False).dtype == torch.int32

@@ -7,9 +7,14 @@ kernels: A (and the output) are physically padded so that every expert starts at
 ``block_m`` rows; ``size_per_group`` holds the real row counts.  Rows in the padding are not
 written.
 
-``grouped_layout`` is what the reference forwards to ``deep_gemm``; it is redundant with
-``size_per_group`` and ``block_m``, so it is accepted and only shape-checked.  The psum form
-(``use_psum_layout=True``) describes the same placement and takes the same path.
+``grouped_layout`` is what the reference forwards to ``deep_gemm``.  When the caller leaves it out it is
+implied by ``size_per_group`` and ``block_m`` (the reference builds it from them).  When the caller passes
+one, the valid rows of every expert are taken from it, on the device and without a host round trip:
+the per-row form ``[M_padded]`` (expert id per row, -1 on padding rows) is counted per expert, the psum form
+``[G]`` (``use_psum_layout=True``: end offset of every expert's valid rows, starts aligned up to ``block_m``)
+is differenced.  Both forms place expert g after expert g-1, each at the next multiple of ``block_m``, as
+``make_deep_gemm_grouped_layout`` / ``make_deep_gemm_psum_layout`` build them; a per-row layout that lists
+experts out of ascending order is not supported.
 """
 from __future__ import annotations
 
@@ -39,7 +44,26 @@ def _check_contiguous_layout(a: torch.Tensor, b: torch.Tensor, size_per_group: t
         want = g if use_psum_layout else m
         if grouped_layout.dim() != 1 or grouped_layout.shape[0] != want:
             raise ValueError(f"grouped_layout must have {want} entries")
+        if grouped_layout.dtype not in (torch.int32, torch.int64):
+            raise ValueError("grouped_layout must be an int32 or int64 tensor")
     return m, n, k, g
+
+
+def sizes_from_layout(grouped_layout: torch.Tensor, num_groups: int, block_m: int, use_psum_layout: bool) -> torch.Tensor:
+    """Valid rows per expert as an explicit layout states them (int32 ``[G]``, on the layout's device, no sync).
+
+    psum form (reference gemm/layout.py:100-119): ``ends[g] = start[g] + size[g]`` with
+    ``start[g] = ceil(ends[g-1] / block_m) * block_m`` and ``start[0] = 0``.  Per-row form (gemm/layout.py:73-97):
+    the number of rows that carry expert id g.
+    """
+    lay = grouped_layout.to(torch.int64)
+    if use_psum_layout:
+        prev = torch.cat([lay.new_zeros(1), lay[:-1]])
+        starts = (prev + (block_m - 1)) // block_m * block_m
+        return (lay - starts).to(torch.int32)
+    counts = torch.zeros(num_groups + 1, dtype=torch.int64, device=lay.device)
+    counts.scatter_add_(0, lay + 1, torch.ones_like(lay))
+    return counts[1:].to(torch.int32)
 
 
 def m_grouped_bf16_nt_contiguous(a: torch.Tensor, b: torch.Tensor, size_per_group: torch.Tensor, *,
@@ -55,7 +79,8 @@ def m_grouped_bf16_nt_contiguous(a: torch.Tensor, b: torch.Tensor, size_per_grou
     _native.require_gpu(a, b, out)
     if not (a.is_contiguous() and b.is_contiguous() and out.is_contiguous()):
         raise ValueError("a, b and out must be contiguous")
-    sizes, is64 = _sizes_on_device(size_per_group, a.device)
+    placed = size_per_group if grouped_layout is None else sizes_from_layout(grouped_layout, g, block_m, use_psum_layout)
+    sizes, is64 = _sizes_on_device(placed, a.device)
     _native.call("tgg_m_grouped_gemm_padded", a.data_ptr(), b.data_ptr(), out.data_ptr(), sizes.data_ptr(), is64, g,
                  m, n, k, int(block_m), _native.BF16, -1, _native.stream_of(a))
     return out
@@ -101,7 +126,8 @@ def m_grouped_fp8_nt_contiguous(a: Tuple[torch.Tensor, torch.Tensor], b: Tuple[t
     if sa.stride() != (1, m) and kb > 1:
         sa = sa.t().contiguous().t()
     sb = b_scale.to(torch.float32).contiguous()
-    sizes, is64 = _sizes_on_device(size_per_group, a_codes.device)
+    placed = size_per_group if grouped_layout is None else sizes_from_layout(grouped_layout, g, block_m, use_psum_layout)
+    sizes, is64 = _sizes_on_device(placed, a_codes.device)
     _native.call("tgg_m_grouped_gemm_fp8_block", a_codes.data_ptr(), sa.data_ptr(), b_codes.data_ptr(),
                  sb.data_ptr(), out.data_ptr(), sizes.data_ptr(), is64, g, m, n, k, int(block_m), 1, -1,
                  _native.stream_of(a_codes))
