@@ -94,9 +94,16 @@ static int tile_order_host(const GemmParams& p, int grid, int split, int64_t* ou
   for (int b = 0; b < grid; ++b) {
     const TileWalk w = sched_walk_of(total, split != 0, grid, b);
     int64_t pos = 0;
+    int g_prev = -1;  // the kernels pass the previous tile's group as a search hint: it must not change the answer
     for (int64_t id = w.first; id < w.end; id += w.stride, ++pos) {
+      const Tile tl = sched_tile<BM, BN>(p, *t, id);
+      const Tile th = sched_tile<BM, BN>(p, *t, id, g_prev);
+      if (th.g != tl.g || th.row0 != tl.row0 || th.rows != tl.rows || th.n0 != tl.n0 || th.k0 != tl.k0 || th.k1 != tl.k1) {
+        delete t;
+        return set_error("hinted tile lookup differs at tile %lld (hint %d)", (long long)id, g_prev);
+      }
+      g_prev = tl.g;
       if (n < capacity) {
-        const Tile tl = sched_tile<BM, BN>(p, *t, id);
         int64_t* r = out + n * 6;
         r[0] = b; r[1] = pos; r[2] = tl.g; r[3] = tl.row0; r[4] = tl.rows; r[5] = tl.n0;
       }

@@ -48,10 +48,20 @@ template <> struct Out16<DT_F16> {
   }
 };
 
+// Two fp32 -> one dword of two 16-bit outputs (first value in the low half), round to nearest even.  Written
+// as a vector conversion so that it becomes one packed convert instead of two converts, a shift and an or.
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+template <int DT> TGG_DEV uint32_t pack2(float a, float b) {
+  const f32x2_t v = {a, b};
+  if (DT == DT_BF16) return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+}
 template <int DT> TGG_DEV uint2 pack4(float a, float b, float c, float d) {
   uint2 r;
-  r.x = (uint32_t)Out16<DT>::cvt(a) | ((uint32_t)Out16<DT>::cvt(b) << 16);
-  r.y = (uint32_t)Out16<DT>::cvt(c) | ((uint32_t)Out16<DT>::cvt(d) << 16);
+  r.x = pack2<DT>(a, b);
+  r.y = pack2<DT>(c, d);
   return r;
 }
 

@@ -68,6 +68,14 @@ TGG_DEV void store_c(i32x4_t* dst, i32x4_t v, int nt) {
   else *dst = v;
 }
 
+// The same through an address that is known to be global memory (an integer turned into a generic pointer would
+// be stored through the flat path, which also counts against the LDS counter).
+TGG_DEV void store_c_global(uint64_t addr, i32x4_t v, int nt) {
+  typedef __attribute__((address_space(1))) i32x4_t* gptr_t;
+  if (nt) __builtin_nontemporal_store(v, (gptr_t)addr);
+  else *(gptr_t)addr = v;
+}
+
 template <int BM_, int BN_, int WM_, int WN_>
 struct FastCfg {
   static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
@@ -228,13 +236,21 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   const TileWalk walk = sched_walk(num_tiles, LAYOUT != LAYOUT_TN && p.tile_split);
   TileIo feed;
   int64_t feed_id;
+  // The tile the feed last looked up is kept: it is the one the multiplying loop asks for a little later, which
+  // saves that loop the lookup (a chain of dependent LDS reads right before a tile's first multiplies).
+  Tile seen;
+  int64_t seen_id = -1;
+  int seen_g = -1;
   auto feed_seek = [&](int64_t id) {
     feed.kt_n = 0;
     feed.issued = 0;
     feed.a_base = feed.b_base = (uint64_t)p.A;
     feed.a_rem = feed.b_rem = feed.a_off = feed.b_off = 0;
     for (; id < walk.end; id += walk.stride) {
-      const Tile tt = sched_tile<C::BM, C::BN>(p, sched, id);
+      const Tile tt = sched_tile<C::BM, C::BN>(p, sched, id, seen_g);
+      seen = tt;
+      seen_id = id;
+      seen_g = tt.g;
       if (slabs_of(tt) > 0) {
         feed = make_io(tt);
         break;
@@ -312,16 +328,26 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   for (int j = 0; j < C::TN; ++j) fb[0][j] = load_b(smem, 0, j);
   int ring = 0;
 
+  // The accumulators start at zero and every epilogue path below clears each strip's registers right after it
+  // has converted them: those moves then sit in the epilogue's LDS waits instead of in front of the next tile's
+  // first multiplies.
+  f32x4_t acc[C::TM][C::TN];
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+  auto clear_strip = [&](int i) {
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+  };
+
   for (int64_t tile_id = walk.first; tile_id < walk.end; tile_id += walk.stride) {
-    const Tile cur = sched_tile<C::BM, C::BN>(p, sched, tile_id);
+    const Tile cur = tile_id == seen_id ? seen : sched_tile<C::BM, C::BN>(p, sched, tile_id);
     const int kt_n = __builtin_amdgcn_readfirstlane(slabs_of(cur));
-    f32x4_t acc[C::TM][C::TN];
-#pragma unroll
-    for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-      for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
 
     // Half a K step: the multiplies of row blocks [h TM/2, (h+1) TM/2) with fragment set `cur_set`.  Meanwhile
     // fragments of K step ks_next of the slab at s_next are read into the other set:
@@ -450,6 +476,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
           }
           *(uint32_t*)(stage_c + e16 * C::EPI_PITCH + 16 * j + 4 * eg) = w;
         }
+        clear_strip(i);
         const i32x4_t v = *(const i32x4_t*)(stage_c + st_row * C::EPI_PITCH + st_chunk * 16);
         if (col_ok && wm0 + 16 * i + st_row < cur.rows)
           store_c((i32x4_t*)(q_tile + (int64_t)(16 * i + st_row) * p.N + st_chunk * 16), v, p.store_nt);
@@ -463,12 +490,42 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
     constexpr int CPS = 2 * C::TN;        // 16-byte chunks per staged row
     constexpr int PASSES = 16 * CPS / 64;  // wave-wide reads per strip
     static_assert(16 * CPS % 64 == 0, "a strip is read back by whole waves");
+    // Tiles that lie wholly inside the output (all but the last row tile of a group and a ragged last column
+    // tile) take a path without per-store bounds checks: a wave-uniform base per strip plus a 32-bit lane offset.
+    const bool full = cur.rows >= C::BM && cur.n0 + C::BN <= p.N;
+    if (full) {
+      const uint64_t base = uniform64((uint64_t)c_tile);
+      const uint32_t strip_bytes = (uint32_t)__builtin_amdgcn_readfirstlane(16 * p.N * 2);
+      uint32_t voff[PASSES];
+#pragma unroll
+      for (int it = 0; it < PASSES; ++it) {
+        const int idx = it * 64 + el, r = idx / CPS, ch = idx % CPS;
+        voff[it] = (uint32_t)(r * p.N * 2 + ch * 16);
+      }
+#pragma unroll
+      for (int i = 0; i < C::TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j)
+          *(uint2*)(stage_c + e16 * C::EPI_PITCH + (16 * j + 4 * eg) * 2) =
+              pack4<DT>(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+        clear_strip(i);
+        const uint64_t strip = base + (uint64_t)i * strip_bytes;
+#pragma unroll
+        for (int it = 0; it < PASSES; ++it) {
+          const int idx = it * 64 + el, r = idx / CPS, ch = idx % CPS;
+          const i32x4_t v = *(const i32x4_t*)(stage_c + r * C::EPI_PITCH + ch * 16);
+          store_c_global(strip + voff[it], v, p.store_nt);
+        }
+      }
+      continue;
+    }
 #pragma unroll
     for (int i = 0; i < C::TM; ++i) {
 #pragma unroll
       for (int j = 0; j < C::TN; ++j)
         *(uint2*)(stage_c + e16 * C::EPI_PITCH + (16 * j + 4 * eg) * 2) =
             pack4<DT>(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+      clear_strip(i);
 #pragma unroll
       for (int it = 0; it < PASSES; ++it) {
         const int idx = it * 64 + el, r = idx / CPS, ch = idx % CPS;

@@ -127,8 +127,11 @@ TGG_HD void sched_split(int r, int rows_m, int tiles_n, int nc, int& mt, int& nt
   nt = c * nc + (q - mt * width);
 }
 
+// g_hint: a group at or before the tile's group, if the caller knows one (a workgroup's walk visits tiles in
+// increasing order, and within a column chunk their groups never decrease): the lookup then checks the hinted
+// group and its successor before it falls back to the binary search, each probe being a dependent LDS read.
 template <int BM, int BN, class Table>
-TGG_HD Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id) {
+TGG_HD Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id, int g_hint = -1) {
   Tile r;
   const int tiles_n = (p.N + BN - 1) / BN;
   const int nc = sched_chunk_width(tiles_n, p.n_chunk);
@@ -151,6 +154,12 @@ TGG_HD Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id) {
   sched_split(tid32, t.tile0[p.G], tiles_n, nc, mt_glob, nt);
   r.n0 = nt * BN;
   int lo = 0, hi = p.G;  // last g with tile0[g] <= mt_glob
+  if (g_hint >= 0 && g_hint < p.G && t.tile0[g_hint] <= mt_glob) {
+    lo = g_hint;
+    if (t.tile0[lo + 1] > mt_glob) hi = lo + 1;            // tile0 has G + 1 entries
+    else if (lo + 2 <= p.G && t.tile0[lo + 2] > mt_glob) { lo = lo + 1; hi = lo + 1; }
+    else lo = lo + 1;                                      // further on: search [lo, G)
+  }
   while (hi - lo > 1) {
     const int mid = (lo + hi) >> 1;
     if (t.tile0[mid] <= mt_glob) lo = mid; else hi = mid;
