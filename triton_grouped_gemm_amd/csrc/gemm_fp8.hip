@@ -136,6 +136,10 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
   const TileWalk walk = sched_walk(num_tiles, false);
   TileIo feed;
   int64_t feed_id;
+  // The multiplying loop looks every tile up one tile ahead (it needs the tile's weight scales early); the feed
+  // reaches that tile later and reuses the lookup instead of repeating its chain of dependent LDS reads.
+  Tile nt;
+  int64_t nt_id = -1;
   auto feed_seek = [&](int64_t id) {
     feed.kt_n = 0;
     feed.issued = 0;
@@ -143,7 +147,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
     feed.a_left = feed.b_left = 0;
     feed.s_bytes = 0;
     for (; id < walk.end; id += walk.stride) {
-      const Tile tt = sched_tile<C::BM, C::BN>(p, sched, id);
+      const Tile tt = id == nt_id ? nt : sched_tile<C::BM, C::BN>(p, sched, id);
       if (slabs_of(tt) > 0) {
         feed = make_io(tt);
         break;
@@ -221,7 +225,6 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
   load_frag(smem + wm0 * 128, fax);
   int ring = 0;
 
-  Tile nt;
   float sbv_next = 0.f;
   if (walk.first < walk.end) {
     nt = sched_tile<C::BM, C::BN>(p, sched, walk.first);
@@ -233,6 +236,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
     float sbv = sbv_next;
     if (tile_id + walk.stride < walk.end) {
       nt = sched_tile<C::BM, C::BN>(p, sched, tile_id + walk.stride);
+      nt_id = tile_id + walk.stride;
       sbv_next = load_sbv(nt);
     }
     f32x16_t acc[C::TM][C::TN];
