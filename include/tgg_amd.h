@@ -154,7 +154,7 @@ int tgg_debug_tile_order(const int64_t* sizes, int G, int mode, int64_t m_total,
  *   "variant"       int  tile configuration of the tuned 16-bit kernels (0 = 256x256 default, 1 = 256x128)
  *   "tile_split"    0/1  16-bit M-grouped: per-XCD contiguous tile ranges (default 1) or interleaved sweeps
  *   "n_chunk"       int  column tiles per chunk of the tile order (0 = automatic, at most eight)
- *   "store_nt"      0/1  write the output with non-temporal stores (default 0) */
+ *   "store_nt"      0/1  write the output with non-temporal stores (default 1) */
 int tgg_set_option(const char* key, int value);
 const char* tgg_last_error(void);
 int tgg_version(void);

@@ -13,7 +13,7 @@ namespace tgg {
 static thread_local char g_err[512] = "";
 static int g_force_generic = 0;
 static int g_tile_split = 1;
-static int g_store_nt = 0;
+static int g_store_nt = 1;
 static int g_n_chunk = 0;
 
 int set_error(const char* fmt, ...) {

@@ -24,6 +24,15 @@ TGG_DEV void copy_b128_to_lds(i32x4_t rsrc, uint32_t lds_addr, int voff) {
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
 }
 
+// Output store of the tuned kernels; dst is global memory.  nt = non-temporal: the output is written once and
+// not read again by the kernel, and with the nt bit the lines do not compete with the operand panels that the
+// other CUs of the XCD keep re-reading from L2 (+4 % on a store-heavy shape, K = 768).  The bit is set through
+// the instruction text: the compiler's non-temporal store builtin did not have that effect here.
+TGG_DEV void store_c(i32x4_t* dst, i32x4_t v, int nt) {
+  if (nt) asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(dst), "v"(v) : "memory");
+  else *(__attribute__((address_space(1))) i32x4_t*)(uint64_t)dst = v;
+}
+
 // Pins a wave-uniform 64-bit value to a scalar register pair.
 TGG_DEV uint64_t uniform64(uint64_t v) {
   const uint32_t lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)v);

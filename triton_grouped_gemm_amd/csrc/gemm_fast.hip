@@ -62,20 +62,6 @@ template <int DT> TGG_DEV float from16(uint16_t h) {
   return (float)__builtin_bit_cast(_Float16, h);
 }
 
-// Output store; nt = streaming hint (the output is written once and not read again by this kernel).
-TGG_DEV void store_c(i32x4_t* dst, i32x4_t v, int nt) {
-  if (nt) __builtin_nontemporal_store(v, dst);
-  else *dst = v;
-}
-
-// The same through an address that is known to be global memory (an integer turned into a generic pointer would
-// be stored through the flat path, which also counts against the LDS counter).
-TGG_DEV void store_c_global(uint64_t addr, i32x4_t v, int nt) {
-  typedef __attribute__((address_space(1))) i32x4_t* gptr_t;
-  if (nt) __builtin_nontemporal_store(v, (gptr_t)addr);
-  else *(gptr_t)addr = v;
-}
-
 template <int BM_, int BN_, int WM_, int WN_>
 struct FastCfg {
   static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
@@ -479,7 +465,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
         clear_strip(i);
         const i32x4_t v = *(const i32x4_t*)(stage_c + st_row * C::EPI_PITCH + st_chunk * 16);
         if (col_ok && wm0 + 16 * i + st_row < cur.rows)
-          store_c((i32x4_t*)(q_tile + (int64_t)(16 * i + st_row) * p.N + st_chunk * 16), v, p.store_nt);
+          store_c((i32x4_t*)(q_tile + (int64_t)(16 * i + st_row) * p.N + st_chunk * 16), v, 0);  // 64-byte row segments: half lines do worse non-temporally
         const int row = wm0 + 16 * i + e16;
         if ((wn & 1) == 0 && eg == 0 && row < cur.rows && cur.n0 + wn0 < p.N)
           p.q_scales[(c_row0 + row) * p.q_rs + (int64_t)blk * p.q_bs] = amax / fmax_;
@@ -514,7 +500,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
         for (int it = 0; it < PASSES; ++it) {
           const int idx = it * 64 + el, r = idx / CPS, ch = idx % CPS;
           const i32x4_t v = *(const i32x4_t*)(stage_c + r * C::EPI_PITCH + ch * 16);
-          store_c_global(strip + voff[it], v, p.store_nt);
+          store_c((i32x4_t*)(strip + voff[it]), v, p.store_nt);
         }
       }
       continue;
