@@ -1,0 +1,73 @@
+"""Randomised shapes: the tuned kernels against the generic kernel, bit for bit.
+
+Both kernels accumulate every output in fp32 over K in ascending order, in 32-deep steps, and round once, so they
+agree exactly; the generic kernel is checked against the CPU oracle elsewhere
+(test_gpu_bf16.py runs every case through both).  What this adds is breadth over group counts, empty groups,
+ragged sizes, N and K tails, both 16-bit types and both size dtypes for the three GEMM kinds.
+"""
+import random
+
+import pytest
+import torch
+
+from triton_grouped_gemm_amd import _native
+from triton_grouped_gemm_amd.gemm.BF16.k_grouped_gemm_TMA import k_grouped_gemm
+from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm_masked_TMA import m_grouped_gemm_masked
+from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm_TMA import m_grouped_gemm
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def dev():
+    return torch.device("cuda:0")
+
+
+def _both(fn):
+    _native.set_option("force_generic", 1)
+    try:
+        ref = fn()
+    finally:
+        _native.set_option("force_generic", 0)
+    out = fn()
+    torch.cuda.synchronize()
+    return out, ref
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_tuned_equals_generic_on_random_shapes(dev, seed):
+    rng = random.Random(1000 + seed)
+    for case in range(15):
+        G = rng.choice([1, 2, 3, 7, 16, 33, 128, 200, 384])
+        sizes = [rng.choice([0, 0, 1, 5, 64, 100, 128, 255, 256, 257, 300, 511, 512, 700]) for _ in range(G)]
+        if G > 64:
+            sizes = [s if rng.random() < 0.3 else 0 for s in sizes]
+        M = sum(sizes)
+        N, K = 8 * rng.randint(1, 130), 8 * rng.randint(1, 70)
+        dt = rng.choice([torch.bfloat16, torch.float16])
+        st = torch.tensor(sizes, dtype=rng.choice([torch.int32, torch.int64]), device=dev)
+        torch.manual_seed(seed * 100 + case)
+        kind = case % 3
+        if kind == 0 and M > 0:
+            tb = rng.random() < 0.5
+            a = (torch.randn(M, K, device=dev) * K ** -0.5).to(dt)
+            b = torch.randn((G, N, K) if tb else (G, K, N), device=dev).to(dt)
+            out, ref = _both(lambda: m_grouped_gemm(a, b, st, tb))
+        elif kind == 1 and M > 0:
+            Md = 8 * rng.randint(1, 80)
+            a = torch.randn(M, Md, device=dev).to(dt)
+            b = torch.randn(M, N, device=dev).to(dt)
+            out, ref = _both(lambda: k_grouped_gemm(a, b, st))
+        else:
+            m_max = 128 * rng.randint(1, 4)
+            mm = torch.tensor([rng.randint(0, m_max) for _ in range(G)], dtype=torch.int32, device=dev)
+            a = (torch.randn(G * m_max, K, device=dev) * K ** -0.5).to(dt)
+            b = torch.randn(G, N, K, device=dev).to(dt)
+
+            def masked():
+                o = torch.full((G * m_max, N), 7.0, dtype=dt, device=dev)
+                m_grouped_gemm_masked(a, b, o, mm, m_max)
+                return o
+
+            out, ref = _both(masked)
+        assert torch.equal(out, ref), f"seed {seed} case {case} kind {kind} G={G} N={N} K={K} {dt}"
