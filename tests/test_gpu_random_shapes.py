@@ -71,3 +71,29 @@ def test_tuned_equals_generic_on_random_shapes(dev, seed):
 
             out, ref = _both(masked)
         assert torch.equal(out, ref), f"seed {seed} case {case} kind {kind} G={G} N={N} K={K} {dt}"
+
+
+@pytest.mark.parametrize("G,per_group,N,K", [(8, 16, 1024, 512), (8, 300, 1024, 512), (4, 64, 264, 136), (64, 700, 512, 256)])
+def test_tile_configurations_agree(dev, G, per_group, N, K):
+    """The tuned 16-bit kernels pick narrow (256x128) tiles on the device when all of them fit one round of
+    workgroups and wide (256x256) tiles otherwise; forcing either gives the same bits as the choice and as the
+    generic kernel (the cases straddle the switch: 8 groups x 8 narrow column tiles fit, 64 x 3 x 4 do not)."""
+    rng = random.Random(G * 1000 + per_group)
+    sizes = [rng.randint(0, per_group) for _ in range(G)]
+    st = torch.tensor(sizes, dtype=torch.int32, device=dev)
+    torch.manual_seed(G + per_group)
+    a = (torch.randn(sum(sizes), K, device=dev) * K ** -0.5).to(torch.bfloat16)
+    b = torch.randn(G, N, K, device=dev).to(torch.bfloat16)
+    ak, bk = torch.randn(sum(sizes), 264, device=dev).to(torch.bfloat16), torch.randn(sum(sizes), N, device=dev).to(torch.bfloat16)
+    _native.set_option("force_generic", 1)
+    try:
+        ref, refk = m_grouped_gemm(a, b, st, True), k_grouped_gemm(ak, bk, st)
+    finally:
+        _native.set_option("force_generic", 0)
+    try:
+        for v in (0, 1, 2):  # chosen on the device, always narrow, always wide
+            _native.set_option("variant", v)
+            assert torch.equal(m_grouped_gemm(a, b, st, True), ref), v
+            assert torch.equal(k_grouped_gemm(ak, bk, st), refk), v
+    finally:
+        _native.set_option("variant", 0)

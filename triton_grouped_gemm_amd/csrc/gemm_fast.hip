@@ -82,16 +82,17 @@ struct FastCfg {
   static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
 };
 
-template <class C, int DT, int LAYOUT, bool QUANT>
-__global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams p) {
+// The whole kernel but for the group table, which the caller has built at byte SCHED_AT of the workgroup's LDS
+// (C::SCHED_OFF unless two tile configurations share one kernel, see gemm_fast_auto_kernel).
+template <class C, int DT, int LAYOUT, bool QUANT, int SCHED_AT>
+TGG_DEV void gemm_fast_body(const GemmParams& p) {
   constexpr bool A_KMAJOR = LAYOUT != LAYOUT_TN;
   constexpr bool B_KMAJOR = LAYOUT == LAYOUT_NT;
   typedef Operand<C::BM, A_KMAJOR> OpA;
   typedef Operand<C::BN, B_KMAJOR> OpB;
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::SCHED_OFF);
-  sched_init<C::BM>(p, sched);
+  const auto& sched = *reinterpret_cast<const SchedTableT<kFastMaxGroups>*>(smem + SCHED_AT);
   const int64_t num_tiles = sched_num_tiles<C::BM, C::BN>(p, sched);
 
   const uint32_t smem_addr = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
@@ -525,30 +526,75 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
 }
 
 template <class C, int DT, int LAYOUT, bool QUANT>
-int launch_cfg(const GemmParams& p, hipStream_t s) {
-  static bool attr_set[64] = {false};
-  int dev = 0;
-  (void)hipGetDevice(&dev);
-  auto kern = gemm_fast_kernel<C, DT, LAYOUT, QUANT>;
-  if (dev >= 0 && dev < 64 && !attr_set[dev]) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM_BYTES) != hipSuccess)
+__global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams p) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  sched_init<C::BM>(p, *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::SCHED_OFF));
+  gemm_fast_body<C, DT, LAYOUT, QUANT, C::SCHED_OFF>(p);
+}
+
+// Two tile configurations in one kernel, chosen per launch from the group sizes, which only the device knows:
+// the narrow tiles (half the columns) when all of them fit into a single round of the persistent workgroups
+// -- twice as many workgroups then have work, and a narrow tile costs about 0.7 of a wide one -- and the wide
+// tiles otherwise.  Both use BM-row tiles, so one group table serves both; it sits where the wide configuration
+// keeps it, past everything the narrow one touches.
+template <class CW, class CN, int DT, int LAYOUT>
+__global__ __launch_bounds__(CW::THREADS) void gemm_fast_auto_kernel(const GemmParams p) {
+  static_assert(CW::BM == CN::BM && CW::THREADS == CN::THREADS, "one group table, one launch shape");
+  static_assert(CN::SMEM_BYTES <= CW::SCHED_OFF, "the narrow configuration must not reach the shared group table");
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + CW::SCHED_OFF);
+  sched_init<CW::BM>(p, sched);
+  if (__builtin_expect(sched_num_tiles<CN::BM, CN::BN>(p, sched) > (int64_t)gridDim.x, 1))
+    gemm_fast_body<CW, DT, LAYOUT, false, CW::SCHED_OFF>(p);
+  else
+    gemm_fast_body<CN, DT, LAYOUT, false, CW::SCHED_OFF>(p);
+}
+
+template <class Kern>
+int launch_kernel(Kern kern, int smem_bytes, int threads, bool& attr_done, const GemmParams& p, hipStream_t s, const char* what) {
+  if (!attr_done) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem_bytes) != hipSuccess)
       return check_launch("hipFuncSetAttribute(gemm_fast)");
-    attr_set[dev] = true;
+    attr_done = true;
   }
   int grid = num_cus();
   if (p.grid_limit > 0 && p.grid_limit < grid) grid = p.grid_limit;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::THREADS), C::SMEM_BYTES, s, p);
-  return check_launch("gemm_fast");
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(threads), smem_bytes, s, p);
+  return check_launch(what);
+}
+
+// The attribute is per device: one flag per device ordinal and kernel.
+inline bool& attr_flag(bool (&flags)[64]) {
+  static bool other = false;
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  if (dev < 0 || dev >= 64) { other = false; return other; }
+  return flags[dev];
+}
+
+template <class C, int DT, int LAYOUT, bool QUANT>
+int launch_cfg(const GemmParams& p, hipStream_t s) {
+  static bool attr_set[64] = {false};
+  return launch_kernel(gemm_fast_kernel<C, DT, LAYOUT, QUANT>, C::SMEM_BYTES, C::THREADS, attr_flag(attr_set), p, s, "gemm_fast");
+}
+
+template <class CW, class CN, int DT, int LAYOUT>
+int launch_auto(const GemmParams& p, hipStream_t s) {
+  static bool attr_set[64] = {false};
+  return launch_kernel(gemm_fast_auto_kernel<CW, CN, DT, LAYOUT>, CW::SMEM_BYTES, CW::THREADS, attr_flag(attr_set), p, s, "gemm_fast");
 }
 
 int g_variant = 0;
 
 template <int DT, int LAYOUT>
 int launch_variant(const GemmParams& p, hipStream_t s) {
+  typedef FastCfg<256, 256, 2, 4> Wide;
+  typedef FastCfg<256, 128, 2, 4> Narrow;
   switch (g_variant) {
     default:
-    case 0: return launch_cfg<FastCfg<256, 256, 2, 4>, DT, LAYOUT, false>(p, s);
-    case 1: return launch_cfg<FastCfg<256, 128, 2, 4>, DT, LAYOUT, false>(p, s);
+    case 0: return launch_auto<Wide, Narrow, DT, LAYOUT>(p, s);
+    case 1: return launch_cfg<Narrow, DT, LAYOUT, false>(p, s);
+    case 2: return launch_cfg<Wide, DT, LAYOUT, false>(p, s);
   }
 }
 
