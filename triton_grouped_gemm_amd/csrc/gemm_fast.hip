@@ -388,6 +388,39 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
       __builtin_amdgcn_sched_barrier(0);
     };
 
+    // A wave whose whole block of the tile lies beyond the group's rows (a group of at most BM / WM rows leaves
+    // the lower waves without work) or beyond N multiplies nothing: it keeps its share of the copy stream and the
+    // barriers going, leaves the matrix pipe to the wave it shares a SIMD with, and ends with the fragment reads
+    // the next tile expects.  Its accumulators are zero and stay zero, and it has nothing to store.
+    if (!QUANT && LAYOUT != LAYOUT_TN && (wm0 >= cur.rows || cur.n0 + wn0 >= p.N)) {
+      for (int kt = 0; kt < kt_n; ++kt) {
+#pragma unroll
+        for (int k = NC / 2; k < NC; ++k) {
+          copy_k(sc, k);
+          __builtin_amdgcn_s_sleep(1);  // paced: the address unit's queue is shared with the working waves
+        }
+        sc_next = begin_slab(ring & 1);
+        wait_vmcnt<0>();
+        __syncthreads();
+        sc = sc_next;
+#pragma unroll
+        for (int k = 0; k < NC / 2; ++k) {
+          copy_k(sc, k);
+          __builtin_amdgcn_s_sleep(1);
+        }
+        ++ring;
+      }
+      if (kt_n > 0) {
+        const char* sn = smem + (ring & 1) * C::STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < C::TM - 1; ++i) fa[i] = load_a(sn, 0, i);
+        fa_last[0] = load_a(sn, 0, C::TM - 1);
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) fb[0][j] = load_b(sn, 0, j);
+      }
+      continue;
+    }
+
     for (int kt = 0; kt < kt_n; ++kt) {
       const char* sa = smem + (ring & 1) * C::STAGE_BYTES;
       const char* sn = smem + ((ring + 1) & 1) * C::STAGE_BYTES;
