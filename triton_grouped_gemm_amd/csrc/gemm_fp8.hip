@@ -3,7 +3,9 @@
 // Same skeleton as the 16-bit kernels (persistent grouped tiles, one continuous direct-to-LDS slab
 // stream across tiles, swizzled LDS, copies interleaved with multiplies, staged epilogue); a slab is
 // 128 bytes = 128 K values of every row, i.e. exactly one 128-wide scale block.  The contraction runs
-// on v_mfma_f32_32x32x64_f8f6f4.
+// on v_mfma_f32_16x16x128_f8f6f4: one multiply per 16x16 output block and slab, operands swapped as in the
+// 16-bit kernels (a lane ends up with 4 consecutive columns of one row).  The shape is a power decision: with all
+// CUs busy on random operands it buys about 9 % more flops per watt than 32x32x64.
 //
 //   EPI_BLOCK    out[r,n] = sum_kb (sum_{k in kb} a[r,k] b[g,n,k]) * sa[kb,r] * sb[g,n/128,kb]
 //                Every slab is contracted into a fresh partial accumulator that is then folded into
@@ -37,16 +39,16 @@ struct Fp8Cfg {
   static constexpr int SA_BYTES = BM * 4 + 256;  // activation scales of the slab's rows + a sink for spare waves' copies
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES + SA_BYTES;
   static constexpr int NI_A = A_BYTES / 1024, NI_B = B_BYTES / 1024;
-  static constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-  static constexpr int EPI_PITCH = 32 * 2 + 16;  // staged 32x32 output block: row pitch in bytes
-  static constexpr int EPI_WAVE_BYTES = 32 * EPI_PITCH;
+  static constexpr int TM = BM / WM / 16, TN = BN / WN / 16;  // 16x16 blocks per wave
+  static constexpr int EPI_PITCH = TN * 32 + 16;  // staged strip of 16 rows x (16 TN) 16-bit outputs: row pitch in bytes
+  static constexpr int EPI_WAVE_BYTES = 16 * EPI_PITCH;
   static constexpr int SCHED_OFF = 2 * STAGE_BYTES;
   static constexpr int EPI_OFF = SCHED_OFF + (((int)sizeof(SchedTableT<kFastMaxGroups>) + 255) & ~255);
   static constexpr int SMEM_BYTES = EPI_OFF + NWAVES * EPI_WAVE_BYTES;
   static_assert(NI_A % NWAVES == 0 && NI_B % NWAVES == 0, "copies must divide evenly over waves");
   static_assert(NWAVES % 2 == 0 && BM / 64 <= NWAVES, "scale copies: one per wave");
   static_assert((BN / WN) <= 128, "a wave's columns must share one 128-wide weight scale block");
-  static_assert(TN == 2 && TM % 2 == 0, "the cell schedule below alternates two B fragments and two A buffers");
+  static_assert(TM >= 4 && TM % 2 == 0 && TN >= 2, "the block schedule below alternates two A fragments");
   static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
 };
 
@@ -67,7 +69,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm0 = (wave / C::WN) * (C::BM / C::WM);
   const int wn0 = (wave % C::WN) * (C::BN / C::WN);
-  const int l32 = lane & 31, lh = lane >> 5;
+  const int l16 = lane & 15, lg = lane >> 4;
 
   const int64_t ld = KGROUP ? p.k_total : (int64_t)p.K;  // bytes between consecutive rows of A and of B
   const int a_voff = OpA::lane_voff(lane, wave % OpA::NPAT, (int)ld);
@@ -79,21 +81,17 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
   const int kblocks = (p.K + 127) >> 7;
   const int nblocks = (p.N + 127) >> 7;
 
-  // LDS offsets of a lane's 32 bytes of fragment (64-deep MFMA step ks): chunks 4 ks + 2 lh + {0, 1}
-  const int fsw = (l32 / 2) % 8;
-  int rd[2][2];
+  // A fragment of the 16x16x128 multiply is 32 consecutive K values per lane: K = 32 lg + (0..31) of row or
+  // column (block + l16), i.e. chunks 2 lg and 2 lg + 1 of its 128-byte LDS row.
+  const int fsw = (l16 / 2) % 8;
+  int rd[2];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-    for (int h = 0; h < 2; ++h) rd[ks][h] = l32 * 128 + (((4 * ks + 2 * lh + h) ^ fsw) << 4);
-  // both K steps of one 32-row block starting at LDS address q
-  auto load_frag = [&](const char* q, i32x8_t (&f)[2]) {
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      const i32x4_t lo = *(const i32x4_t*)(q + rd[ks][0]);
-      const i32x4_t hi = *(const i32x4_t*)(q + rd[ks][1]);
-      f[ks] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
+  for (int h = 0; h < 2; ++h) rd[h] = l16 * 128 + (((2 * lg + h) ^ fsw) << 4);
+  // the fragment of the 16-row block starting at LDS address q
+  auto load_frag = [&](const char* q) -> i32x8_t {
+    const i32x4_t lo = *(const i32x4_t*)(q + rd[0]);
+    const i32x4_t hi = *(const i32x4_t*)(q + rd[1]);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
 
   // Slab sequence of a tile in scalar registers (see gemm_fast.hip): next slab's start and remaining bytes
@@ -194,13 +192,16 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
     }
   };
 
-  // Software pipeline.  A slab is worked off in TM x 2 cells (32-row block i, 32-column block j), two
-  // 64-deep multiplies each.  The B fragments of both column blocks stay in registers for the slab, the
-  // A fragments of row block i+1 are read during row block i.  Before the last cell (TM-1, 1): wait for
-  // this wave's share of the next slab, workgroup barrier, read the next slab's j = 0 and i = 0
-  // fragments (the registers of the current slab's j = 0 fragments are free by then), then multiply;
-  // the next slab's j = 1 fragments follow during its first cell.  The copies of the slab after the
-  // next one are issued one per multiply from that point on (see gemm_fast.hip for why).
+  // Software pipeline.  A slab is TM x TN multiplies, one per 16x16 block, row block by row block.  The B
+  // fragments of all column blocks stay in registers for the slab; the A fragment of row block i + 1 is read
+  // during row block i (two registers sets alternate).  Before the last row block: wait for this wave's share of
+  // the next slab, workgroup barrier, read the next slab's first A fragment; each of the last row block's
+  // multiplies is followed by the read of the next slab's B fragment into the registers it has just used.  The
+  // copies of the slab after the next one are issued one per multiply from the barrier on: the sooner they are
+  // out, the longer they have to land before the next wait (one per two multiplies measured 3 % slower, two per
+  // multiply 4 % slower: the address unit's queue is short, see gemm_fast.hip).
+  // Block scaling: every multiply starts from zero and its result is folded into the accumulators, scaled, two
+  // multiplies later.
   feed_seek(walk.first);
   {
     const SlabCopy s0 = begin_slab(0);
@@ -220,9 +221,12 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
   };
   copy_at(0);
   copy_at(1);
-  i32x8_t fb0[2], fb1[2], fax[2], fay[2];
-  load_frag(smem + C::A_BYTES + wn0 * 128, fb0);
-  load_frag(smem + wm0 * 128, fax);
+  copy_at(2);
+  copy_at(3);
+  i32x8_t fb[C::TN], fa[2];
+#pragma unroll
+  for (int j = 0; j < C::TN; ++j) fb[j] = load_frag(smem + C::A_BYTES + (wn0 + 16 * j) * 128);
+  fa[0] = load_frag(smem + wm0 * 128);
   int ring = 0;
 
   float sbv_next = 0.f;
@@ -230,6 +234,21 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
     nt = sched_tile<C::BM, C::BN>(p, sched, walk.first);
     sbv_next = load_sbv(nt);
   }
+  // The accumulators start at zero and the epilogue clears every strip right after it has converted it.
+  f32x4_t acc[C::TM][C::TN];
+#pragma unroll
+  for (int i = 0; i < C::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+  auto clear_strip = [&](int i) {
+#pragma unroll
+    for (int j = 0; j < C::TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+  };
+
   for (int64_t tile_id = walk.first; tile_id < walk.end; tile_id += walk.stride) {
     const Tile cur = nt;
     const int kt_n = __builtin_amdgcn_readfirstlane(slabs_of(cur));
@@ -239,134 +258,142 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
       nt_id = tile_id + walk.stride;
       sbv_next = load_sbv(nt);
     }
-    f32x16_t acc[C::TM][C::TN];
-#pragma unroll
-    for (int i = 0; i < C::TM; ++i)
-#pragma unroll
-      for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
+    // block scaling: the products that are still to be folded in when a slab ends (those of its last two
+    // multiplies) are carried into the next slab
+    f32x4_t part[4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    float s_carry = 0.f;
     for (int kt = 0; kt < kt_n; ++kt) {
       const char* sa = smem + (ring & 1) * C::STAGE_BYTES;
       const char* sn = smem + ((ring + 1) & 1) * C::STAGE_BYTES;
       float srow[C::TM];
       if (BLOCK) {
         const float sb_cur = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sbv), kt));
-        const float* ss = (const float*)(sa + C::A_BYTES + C::B_BYTES) + wm0 + l32;
+        const float* ss = (const float*)(sa + C::A_BYTES + C::B_BYTES) + wm0 + l16;
 #pragma unroll
-        for (int i = 0; i < C::TM; ++i) srow[i] = ss[32 * i] * sb_cur;
+        for (int i = 0; i < C::TM; ++i) srow[i] = ss[16 * i] * sb_cur;
       }
-      // one cell: two multiplies, with `mid` run right after the first has been issued; copies k0 and
-      // k0 + 1 of the slab being requested go out after the first and the second multiply
-      auto cell = [&](int i, int j, int k0, const i32x8_t (&fa)[2], const i32x8_t (&fb)[2], auto&& mid) {
-        if (BLOCK) {
-          f32x16_t part = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-          part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[0], fa[0], part, FB, FA, 0, 0, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
-          mid();
-          copy_at(k0);
-          __builtin_amdgcn_sched_barrier(0);
-          part = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[1], fa[1], part, FB, FA, 0, 0, 0, 0);
-          copy_at(k0 + 1);
-          // the empty asm statements pin the scaling between the multiplies of this cell and the next one
-          // (plain arithmetic is otherwise free to drift, which keeps many partial tiles alive at once)
-          asm volatile("" : "+v"(part));
+      SlabCopy scn;
 #pragma unroll
-          for (int e = 0; e < 16; ++e) acc[i][j][e] += part[e] * srow[i];
-          asm volatile("" : "+v"(acc[i][j]));
-        } else {
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[0], fa[0], acc[i][j], FB, FA, 0, 0, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
-          mid();
-          copy_at(k0);
-          __builtin_amdgcn_sched_barrier(0);
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[1], fa[1], acc[i][j], FB, FA, 0, 0, 0, 0);
-          copy_at(k0 + 1);
-        }
+      for (int i = 0; i < C::TM; ++i) {
         __builtin_amdgcn_sched_barrier(0);
-      };
-#pragma unroll
-      for (int i = 0; i < C::TM; i += 2) {
-        // row block i from fax, i + 1 from fay; cell c of the slab issues copies 2 + 2 c and 3 + 2 c
-        cell(i, 0, 2 + 4 * i, fax, fb0, [&] {
-          if (i == 0) load_frag(sa + C::A_BYTES + (wn0 + 32) * 128, fb1);
-          load_frag(sa + (wm0 + 32 * (i + 1)) * 128, fay);
-        });
-        cell(i, 1, 4 + 4 * i, fax, fb1, [&] {});
-        if (i + 2 < C::TM) {
-          cell(i + 1, 0, 6 + 4 * i, fay, fb0, [&] { load_frag(sa + (wm0 + 32 * (i + 2)) * 128, fax); });
-          cell(i + 1, 1, 8 + 4 * i, fay, fb1, [&] {});
+        if (i < C::TM - 1) {
+          fa[(i + 1) & 1] = load_frag(sa + (wm0 + 16 * (i + 1)) * 128);
         } else {
-          SlabCopy scn;
-          cell(i + 1, 0, 6 + 4 * i, fay, fb0, [&] { scn = begin_slab(ring & 1); });  // scalar work under a multiply
           wait_vmcnt<0>();
           if (BLOCK) asm volatile("" : "+v"(sbv_next));  // nothing of this wave is in flight: touching it costs no wait
           __syncthreads();
           sc = scn;
-          load_frag(sn + C::A_BYTES + wn0 * 128, fb0);
-          load_frag(sn + wm0 * 128, fax);
+          fa[0] = load_frag(sn + wm0 * 128);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int jj = 0; jj < C::TN; ++jj) {
+          // snake order over the column blocks, except that the last row block runs forward: its multiplies free
+          // the B registers in the order in which the next slab's first row block needs them
+          const int j = ((i & 1) && i != C::TM - 1) ? C::TN - 1 - jj : jj;
+          const int n = i * C::TN + jj;
+          if (BLOCK) {
+            const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+            part[n & 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], fa[i & 1], zero, FB, FA, 0, 0, 0, 0);
+          } else {
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb[j], fa[i & 1], acc[i][j], FB, FA, 0, 0, 0, 0);
+          }
           __builtin_amdgcn_sched_barrier(0);
-          cell(i + 1, 1, 0, fay, fb1, [&] {});
+          if (i == C::TM - 1) {
+            copy_at(jj);
+            fb[j] = load_frag(sn + C::A_BYTES + (wn0 + 16 * j) * 128);
+          } else {
+            if (n == C::TN * (C::TM - 2) + 1) scn = begin_slab(ring & 1);  // scalar work under a multiply
+            copy_at(C::TN + n);
+          }
+          if (BLOCK) {
+            // fold in the product of the multiply before the previous one (it has had two issue slots to finish;
+            // for n = 0, 1 that is one of the previous slab's last two, scaled with that slab's last row scale).
+            // Four product buffers, indexed by n % 4.  The empty asm statements pin the order (plain arithmetic is
+            // otherwise free to drift, which keeps many products alive at once and spills).
+            constexpr int NB = C::TM * C::TN;
+            static_assert(NB % 4 == 0, "product buffers are numbered per slab");
+            const int pn = (n + NB - 2) % NB;
+            const int pi = pn / C::TN, pjj = pn % C::TN;
+            const int pj = ((pi & 1) && pi != C::TM - 1) ? C::TN - 1 - pjj : pjj;
+            const float sc_prev = n < 2 ? s_carry : srow[pi];
+            const int pb = pn & 3;
+            asm volatile("" : "+v"(part[pb]));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[pi][pj][e] += part[pb][e] * sc_prev;
+            asm volatile("" : "+v"(acc[pi][pj]));
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
+      if (BLOCK) s_carry = srow[C::TM - 1];
       ++ring;
     }
+    if (BLOCK) {
+#pragma unroll
+      for (int q = 1; q >= 0; --q) {
+        constexpr int NB = C::TM * C::TN;
+        const int pn = NB - 1 - q;
+        const int pj = pn % C::TN;  // the last row block runs forward
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[C::TM - 1][pj][e] += part[pn & 3][e] * s_carry;
+      }
+    }
 
-    // Epilogue (see gemm_fast.hip): per-channel scaling happens on the fp32 values before packing.
+    // Epilogue (see gemm_fast.hip): a lane owns row l16 and columns 16 j + 4 lg + (0..3) of each 16-row block i.
+    // One 16-row strip of the wave's columns at a time goes through the wave's LDS staging and leaves as 16-byte
+    // stores that cover whole row segments; per-channel scaling happens on the fp32 values before packing.
     // The lane id passes through an opaque statement so that the address arithmetic below is redone per tile
     // instead of being hoisted: hoisted values would have to live (spilled) across the register-tight main loop,
     // and every reload waits for all outstanding stores.
     int el = lane;
     asm volatile("" : "+v"(el));
-    const int e32 = el & 31, eh = el >> 5;
-    const int st_row = el >> 2, st_chunk = el & 3;
+    const int e16 = el & 15, eg = el >> 4;
     char* const stage = smem + C::EPI_OFF + wave * C::EPI_WAVE_BYTES;
     const int64_t c_row0 = KGROUP ? ((int64_t)cur.g * p.m_total + cur.row0) : cur.row0;
     char* const c_tile = (char*)p.C + ((c_row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2;
-    // channel scales of this lane's rows and columns, fetched up front in a few wide loads
-    float rs[C::TM];
-    f32x4_t cs[C::TN][4];
+    constexpr int CPS = 2 * C::TN;         // 16-byte chunks per staged row
+    constexpr int PASSES = 16 * CPS / 64;  // wave-wide reads per strip
+    static_assert(16 * CPS % 64 == 0, "a strip is read back by whole waves");
+    // channel scales of this lane's columns, fetched up front; those of its rows strip by strip
+    f32x4_t cs[C::TN];
+    const float* sm = nullptr;
     if (EPI == EPI_CHANNEL) {
-      const float* sm = p.scale_m + (KGROUP ? (int64_t)cur.g * p.scale_m_sg : 0) + cur.row0;
-#pragma unroll
-      for (int i = 0; i < C::TM; ++i) {
-        const int m = wm0 + 32 * i + e32;
-        rs[i] = m < cur.rows ? sm[m] : 0.f;
-      }
+      sm = p.scale_m + (KGROUP ? (int64_t)cur.g * p.scale_m_sg : 0) + cur.row0;
       const float* sn = p.scale_n + (int64_t)cur.g * p.N;
 #pragma unroll
-      for (int j = 0; j < C::TN; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = cur.n0 + wn0 + 32 * j + 8 * q + 4 * eh;  // N is a multiple of 8: 4 columns are in or out together
-          const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
-          cs[j][q] = n < p.N ? *(const f32x4_t*)(sn + n) : zero;
-        }
+      for (int j = 0; j < C::TN; ++j) {
+        const int n = cur.n0 + wn0 + 16 * j + 4 * eg;  // N is a multiple of 8: 4 columns are in or out together
+        const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+        cs[j] = n < p.N ? *(const f32x4_t*)(sn + n) : zero;
+      }
     }
 #pragma unroll
     for (int i = 0; i < C::TM; ++i) {
+      float rs = 1.f;
+      if (EPI == EPI_CHANNEL) {
+        const int m = wm0 + 16 * i + e16;
+        rs = m < cur.rows ? sm[m] : 0.f;
+      }
 #pragma unroll
       for (int j = 0; j < C::TN; ++j) {
+        float v[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          float v[4];
+        for (int e = 0; e < 4; ++e) v[e] = acc[i][j][e];
+        if (EPI == EPI_CHANNEL) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * q + e];
-          if (EPI == EPI_CHANNEL) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = v[e] * rs[i] * cs[j][q][e];
-          }
-          *(uint2*)(stage + e32 * C::EPI_PITCH + (8 * q + 4 * eh) * 2) = pack4<OUT>(v[0], v[1], v[2], v[3]);
+          for (int e = 0; e < 4; ++e) v[e] = v[e] * rs * cs[j][e];
         }
-        const bool col_ok = cur.n0 + wn0 + 32 * j + st_chunk * 8 < p.N;
+        *(uint2*)(stage + e16 * C::EPI_PITCH + (16 * j + 4 * eg) * 2) = pack4<OUT>(v[0], v[1], v[2], v[3]);
+      }
+      clear_strip(i);
 #pragma unroll
-        for (int it = 0; it < 2; ++it) {
-          const int r = it * 16 + st_row;
-          const i32x4_t v = *(const i32x4_t*)(stage + r * C::EPI_PITCH + st_chunk * 16);
-          if (col_ok && wm0 + 32 * i + r < cur.rows)
-            *(i32x4_t*)(c_tile + ((int64_t)(32 * i + r) * p.N + 32 * j + st_chunk * 8) * 2) = v;
-        }
+      for (int it = 0; it < PASSES; ++it) {
+        const int idx = it * 64 + el, r = idx / CPS, ch = idx % CPS;
+        const i32x4_t v = *(const i32x4_t*)(stage + r * C::EPI_PITCH + ch * 16);
+        if (cur.n0 + wn0 + ch * 8 < p.N && wm0 + 16 * i + r < cur.rows)
+          store_c((i32x4_t*)(c_tile + ((int64_t)(16 * i + r) * p.N + ch * 8) * 2), v, p.store_nt);
       }
     }
   }
