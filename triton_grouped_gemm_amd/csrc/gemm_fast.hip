@@ -253,8 +253,13 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
     bool tail;  // the tile's last slab, cut short by K
   };
   constexpr int CA = C::NI_A / C::NWAVES, CB = C::NI_B / C::NWAVES, NC = CA + CB;
-  constexpr int SP = (C::TM * C::TN / 2) / (NC / 2);  // multiplies between two copies
-  static_assert(NC % 2 == 0 && SP >= 1, "a slab's copies are spread over the multiplies of two half K steps");
+  // multiplies between two copies: the first half of a slab's copies goes out right after the barrier, one per
+  // multiply (the sooner they are out, the longer they have to land: +1.5-2 % over one per four multiplies;
+  // not so with two token-row operands, where the denser issue measured 1.3 % slower), the second half one per
+  // four multiplies during the following half step (all eight early: -2 %, the address unit's queue is short)
+  constexpr int SP2 = (C::TM * C::TN / 2) / (NC / 2);
+  constexpr int SP1 = LAYOUT == LAYOUT_TN ? SP2 : 1;
+  static_assert(NC % 2 == 0 && SP2 >= 1, "a slab's copies are spread over the multiplies of two half K steps");
   auto begin_slab = [&](int buf) {
     SlabCopy sc;
     const bool live = feed.issued < feed.kt_n;
@@ -291,7 +296,7 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
   //   then wait for this wave's share of slab r+1 and pass the workgroup barrier: slab r+1 is complete and
   //   nobody reads slab r any more, its last fragments are already in registers;
   //   step 1, 2nd half  multiply while reading step 0 of slab r+1 (first the fragments the 1st half skipped).
-  // The copies of slab r+2 (into slab r's buffer) are issued one per SP multiplies during the half step after
+  // The copies of slab r+2 (into slab r's buffer) are issued between the multiplies of the half step after
   // the barrier and the half step after that, which leaves them a whole K step to land before they are waited
   // for.  They are spread out because the texture-address unit takes 16 cycles per copy instruction and its
   // queue is short: a wave that issues its copies back to back sits blocked behind the other waves' copies with
@@ -343,7 +348,7 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
     //   READ_ROLL     A fragment i after the multiplies of row block i;
     //   READ_NONE     nothing (the slab to read from is not complete yet);
     //   READ_CATCH_UP as READ_EARLY, plus the A fragments that the preceding READ_NONE half left out.
-    // Copies [k0, k0 + NC/2) of `sc` are issued one per SP multiplies when k0 >= 0.
+    // Copies [k0, k0 + NC/2) of `sc` are issued between the multiplies when k0 >= 0 (SP1, SP2 above).
     enum { READ_EARLY, READ_ROLL, READ_NONE, READ_CATCH_UP };
     SlabCopy sc_next;
     auto half = [&](int cur_set, int h, const char* s_next, int ks_next, int mode, int k0, bool prepare = false) {
@@ -373,9 +378,10 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
             __builtin_amdgcn_sched_barrier(0);
           }
           if (prepare && n == 1) sc_next = begin_slab(ring & 1);  // scalar work, under the multiplies just issued
-          if (k0 >= 0 && (n + 1) % SP == 0 && (n + 1) / SP <= NC / 2) {
+          const int sp = k0 == 0 ? SP1 : SP2;
+          if (k0 >= 0 && (n + 1) % sp == 0 && (n + 1) / sp <= NC / 2) {
             __builtin_amdgcn_sched_barrier(0);
-            copy_k(sc, k0 + (n + 1) / SP - 1);
+            copy_k(sc, k0 + (n + 1) / sp - 1);
             __builtin_amdgcn_sched_barrier(0);
           }
         }
