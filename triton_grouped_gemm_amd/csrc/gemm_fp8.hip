@@ -266,12 +266,15 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
     for (int kt = 0; kt < kt_n; ++kt) {
       const char* sa = smem + (ring & 1) * C::STAGE_BYTES;
       const char* sn = smem + ((ring + 1) & 1) * C::STAGE_BYTES;
+      // row scales of the slab: read here, multiplied with the weight scale only after the row block's first
+      // multiply has been issued, so that the wait for the reads does not sit in front of the slab's first multiply
       float srow[C::TM];
+      float sb_cur = 0.f;
       if (BLOCK) {
-        const float sb_cur = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sbv), kt));
+        sb_cur = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sbv), kt));
         const float* ss = (const float*)(sa + C::A_BYTES + C::B_BYTES) + wm0 + l16;
 #pragma unroll
-        for (int i = 0; i < C::TM; ++i) srow[i] = ss[16 * i] * sb_cur;
+        for (int i = 0; i < C::TM; ++i) srow[i] = ss[16 * i];
       }
       SlabCopy scn;
 #pragma unroll
@@ -307,6 +310,7 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
             if (n == C::TN * (C::TM - 2) + 1) scn = begin_slab(ring & 1);  // scalar work under a multiply
             copy_at(C::TN + n);
           }
+          if (BLOCK && jj == 0) srow[i] *= sb_cur;
           if (BLOCK) {
             // fold in the product of the multiply before the previous one (it has had two issue slots to finish;
             // for n = 0, 1 that is one of the previous slab's last two, scaled with that slab's last row scale).
