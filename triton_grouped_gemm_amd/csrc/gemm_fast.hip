@@ -14,7 +14,7 @@
 //     workgroup's tiles form one uninterrupted stream: the copies run two slabs ahead of the
 //     multiplies across tile boundaries, and the fragment reads run one K step ahead across the
 //     barrier, so neither the barrier nor the LDS latency behind it leaves the matrix pipe idle.
-//   * A slab's copy instructions are issued one per two multiplies rather than back to back: the
+//   * A slab's copy instructions are issued between multiplies rather than back to back: the
 //     address unit takes 16 cycles per copy and has a short queue, and a wave blocked on that queue
 //     cannot issue its multiplies.
 //   * LDS is XOR-swizzled at 16-byte granularity.  The direct-to-LDS copy is lane-linear on the
@@ -602,12 +602,15 @@ int launch_kernel(Kern kern, int smem_bytes, int threads, bool& attr_done, const
   return check_launch(what);
 }
 
-// The attribute is per device: one flag per device ordinal and kernel.
+// The attribute is per device: one flag per device ordinal and kernel (devices beyond the table set it every time).
 inline bool& attr_flag(bool (&flags)[64]) {
-  static bool other = false;
+  static thread_local bool unlisted;
   int dev = 0;
   (void)hipGetDevice(&dev);
-  if (dev < 0 || dev >= 64) { other = false; return other; }
+  if (dev < 0 || dev >= 64) {
+    unlisted = false;
+    return unlisted;
+  }
   return flags[dev];
 }
 
