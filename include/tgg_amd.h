@@ -151,7 +151,7 @@ int tgg_debug_tile_order(const int64_t* sizes, int G, int mode, int64_t m_total,
 
 /* Library controls (process-wide, meant for tests and tuning; returns 1 for an unknown key):
  *   "force_generic" 0/1  route every GEMM through the shape-agnostic kernel
- *   "variant"       int  tile configuration of the tuned 16-bit kernels: 0 (default) = chosen per launch on the
+ *   "variant"       int  tile configuration of the tuned kernels (16-bit, and FP8 M-grouped): 0 (default) = chosen per launch on the
  *                        device from the group sizes -- 256x128 when all such tiles fit one round of the persistent
  *                        workgroups, 256x256 otherwise; 1 = always 256x128; 2 = always 256x256
  *   "tile_split"    0/1  16-bit M-grouped: per-XCD contiguous tile ranges (default 1) or interleaved sweeps

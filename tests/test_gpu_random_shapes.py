@@ -97,3 +97,38 @@ def test_tile_configurations_agree(dev, G, per_group, N, K):
             assert torch.equal(k_grouped_gemm(ak, bk, st), refk), v
     finally:
         _native.set_option("variant", 0)
+
+
+@pytest.mark.parametrize("G,per_group,N,K", [(4, 128, 1024, 512), (8, 384, 1024, 256), (40, 256, 768, 384)])
+def test_fp8_tile_configurations_agree(dev, G, per_group, N, K):
+    """The FP8 M-grouped kernels make the same choice between 256x128 and 256x256 tiles; either width gives the
+    same bits (block-scaled and per-channel), and the generic kernel agrees."""
+    from triton_grouped_gemm_amd.gemm.deep_gemm_ops import m_grouped_fp8_nt_contiguous
+    from triton_grouped_gemm_amd.gemm.FP8.m_grouped_gemm_channel_expert import gmm_fp8_act_per_channel_w_per_expert
+    from triton_grouped_gemm_amd.quant.fp8_cast import per_block_cast_to_fp8, per_token_cast_to_fp8
+    rng = random.Random(G * 7 + per_group)
+    sizes = [128 * rng.randint(0, per_group // 128) for _ in range(G)]
+    st = torch.tensor(sizes, dtype=torch.int32, device=dev)
+    torch.manual_seed(G)
+    a = torch.randn(max(sum(sizes), 128), K, device=dev).to(torch.bfloat16)[:sum(sizes)]
+    w = torch.randn(G, N, K, device=dev).to(torch.bfloat16)
+    aq, sa = per_token_cast_to_fp8(a, scales_mn_major=True)
+    wq, sb = per_block_cast_to_fp8(w)
+    ca, cb = torch.rand(sum(sizes), 1, device=dev) + 0.5, torch.rand(G * N, device=dev) + 0.5
+
+    def both():
+        return (m_grouped_fp8_nt_contiguous((aq, sa), (wq, sb), st),
+                gmm_fp8_act_per_channel_w_per_expert(aq, ca, wq, cb, st, torch.bfloat16))
+
+    _native.set_option("force_generic", 1)
+    try:
+        ref = both()
+    finally:
+        _native.set_option("force_generic", 0)
+    try:
+        for v in (0, 1, 2):
+            _native.set_option("variant", v)
+            out = both()
+            assert torch.equal(out[0], ref[0]) and torch.equal(out[1], ref[1]), v
+    finally:
+        _native.set_option("variant", 0)

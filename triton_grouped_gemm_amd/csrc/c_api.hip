@@ -52,6 +52,7 @@ int launch_fast_16bit(const GemmParams& p, int dt, int layout, hipStream_t s);
 bool fast_quant_supported(const GemmParams& p, int dt, int layout);
 int launch_fast_16bit_quant(const GemmParams& p, int dt, int layout, hipStream_t s);
 void set_fast_variant(int v);
+void set_fp8_variant(int v);
 
 static bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 
@@ -402,7 +403,7 @@ int tgg_debug_tile_order(const int64_t* sizes, int G, int mode, int64_t m_total,
 
 int tgg_set_option(const char* key, int value) {
   if (key && strcmp(key, "force_generic") == 0) { g_force_generic = value != 0; return 0; }
-  if (key && strcmp(key, "variant") == 0) { set_fast_variant(value); return 0; }
+  if (key && strcmp(key, "variant") == 0) { set_fast_variant(value); set_fp8_variant(value); return 0; }
   if (key && strcmp(key, "tile_split") == 0) { g_tile_split = value != 0; return 0; }
   if (key && strcmp(key, "n_chunk") == 0) { g_n_chunk = value < 0 ? 0 : value; return 0; }
   if (key && strcmp(key, "store_nt") == 0) { g_store_nt = value != 0; return 0; }

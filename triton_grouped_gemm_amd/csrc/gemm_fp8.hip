@@ -53,15 +53,15 @@ struct Fp8Cfg {
 };
 
 // FA / FB: 0 = e4m3fn, 1 = e5m2 (the cbsz / blgp format codes of the f8f6f4 MFMA).
-template <class C, int FA, int FB, int EPI, int OUT, bool KGROUP>
-__global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p) {
+// The whole kernel but for the group table, which the caller has built at byte SCHED_AT of the workgroup's LDS.
+template <class C, int FA, int FB, int EPI, int OUT, bool KGROUP, int SCHED_AT>
+TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   typedef Operand<C::BM, true> OpA;
   typedef Operand<C::BN, true> OpB;
   constexpr bool BLOCK = EPI == EPI_BLOCK;
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::SCHED_OFF);
-  sched_init<C::BM>(p, sched);
+  const auto& sched = *reinterpret_cast<const SchedTableT<kFastMaxGroups>*>(smem + SCHED_AT);
   const int64_t num_tiles = sched_num_tiles<C::BM, C::BN>(p, sched);
 
   const uint32_t smem_addr = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
@@ -219,10 +219,8 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  copy_at(0);
-  copy_at(1);
-  copy_at(2);
-  copy_at(3);
+#pragma unroll
+  for (int k = 0; k < C::TN; ++k) copy_at(k);
   i32x8_t fb[C::TN], fa[2];
 #pragma unroll
   for (int j = 0; j < C::TN; ++j) fb[j] = load_frag(smem + C::A_BYTES + (wn0 + 16 * j) * 128);
@@ -405,28 +403,66 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
 }
 
 template <class C, int FA, int FB, int EPI, int OUT, bool KGROUP>
-int launch_fp8_cfg(const GemmParams& p, hipStream_t s) {
-  static bool attr_set[64] = {false};
+__global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  sched_init<C::BM>(p, *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::SCHED_OFF));
+  gemm_fp8_body<C, FA, FB, EPI, OUT, KGROUP, C::SCHED_OFF>(p);
+}
+
+// Two tile widths in one kernel, chosen per launch on the device (see gemm_fast_auto_kernel in gemm_fast.hip): the
+// narrow tiles when all of them fit one round of the persistent workgroups, the wide ones otherwise.
+template <class CW, class CN, int FA, int FB, int EPI, int OUT>
+__global__ __launch_bounds__(CW::THREADS) void gemm_fp8_auto_kernel(const GemmParams p) {
+  static_assert(CW::BM == CN::BM && CW::THREADS == CN::THREADS, "one group table, one launch shape");
+  static_assert(CN::SMEM_BYTES <= CW::SCHED_OFF, "the narrow configuration must not reach the shared group table");
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + CW::SCHED_OFF);
+  sched_init<CW::BM>(p, sched);
+  if (__builtin_expect(sched_num_tiles<CN::BM, CN::BN>(p, sched) > (int64_t)gridDim.x, 1))
+    gemm_fp8_body<CW, FA, FB, EPI, OUT, false, CW::SCHED_OFF>(p);
+  else
+    gemm_fp8_body<CN, FA, FB, EPI, OUT, false, CW::SCHED_OFF>(p);
+}
+
+template <class Kern>
+int launch_fp8_kernel(Kern kern, int smem_bytes, int threads, bool (&attr_set)[64], const GemmParams& p, hipStream_t s) {
   int dev = 0;
   (void)hipGetDevice(&dev);
-  auto kern = gemm_fp8_kernel<C, FA, FB, EPI, OUT, KGROUP>;
-  if (dev >= 0 && dev < 64 && !attr_set[dev]) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM_BYTES) != hipSuccess)
+  const bool listed = dev >= 0 && dev < 64;
+  if (!listed || !attr_set[dev]) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem_bytes) != hipSuccess)
       return check_launch("hipFuncSetAttribute(gemm_fp8)");
-    attr_set[dev] = true;
+    if (listed) attr_set[dev] = true;
   }
   int grid = num_cus();
   if (p.grid_limit > 0 && p.grid_limit < grid) grid = p.grid_limit;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::THREADS), C::SMEM_BYTES, s, p);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(threads), smem_bytes, s, p);
   return check_launch("gemm_fp8");
 }
 
-typedef Fp8Cfg<256, 256, 2, 4> Fp8Default;
+typedef Fp8Cfg<256, 256, 2, 4> Fp8Wide;
+typedef Fp8Cfg<256, 128, 2, 4> Fp8Narrow;
+
+int g_fp8_variant = 0;  // 0: chosen on the device (M-grouped), 1: narrow, 2: wide
+
+// M-grouped launches choose the tile width on the device; K-grouped ones (tile count known to the host, tile cost
+// set by the group's token count) use the wide tiles.
+template <int FA, int FB, int EPI, int OUT, bool KGROUP>
+int launch_fp8_cfg(const GemmParams& p, hipStream_t s) {
+  static bool attr_auto[64] = {false}, attr_wide[64] = {false}, attr_narrow[64] = {false};
+  if constexpr (!KGROUP) {
+    if (g_fp8_variant == 0)
+      return launch_fp8_kernel(gemm_fp8_auto_kernel<Fp8Wide, Fp8Narrow, FA, FB, EPI, OUT>, Fp8Wide::SMEM_BYTES, Fp8Wide::THREADS, attr_auto, p, s);
+    if (g_fp8_variant == 1)
+      return launch_fp8_kernel(gemm_fp8_kernel<Fp8Narrow, FA, FB, EPI, OUT, false>, Fp8Narrow::SMEM_BYTES, Fp8Narrow::THREADS, attr_narrow, p, s);
+  }
+  return launch_fp8_kernel(gemm_fp8_kernel<Fp8Wide, FA, FB, EPI, OUT, KGROUP>, Fp8Wide::SMEM_BYTES, Fp8Wide::THREADS, attr_wide, p, s);
+}
 
 template <int FA, int FB, bool KGROUP>
 int launch_channel_out(const GemmParams& p, int out_dt, hipStream_t s) {
-  if (out_dt == DT_BF16) return launch_fp8_cfg<Fp8Default, FA, FB, EPI_CHANNEL, DT_BF16, KGROUP>(p, s);
-  if (out_dt == DT_F16) return launch_fp8_cfg<Fp8Default, FA, FB, EPI_CHANNEL, DT_F16, KGROUP>(p, s);
+  if (out_dt == DT_BF16) return launch_fp8_cfg<FA, FB, EPI_CHANNEL, DT_BF16, KGROUP>(p, s);
+  if (out_dt == DT_F16) return launch_fp8_cfg<FA, FB, EPI_CHANNEL, DT_F16, KGROUP>(p, s);
   return set_error("unsupported output dtype code %d", out_dt);
 }
 
@@ -440,6 +476,8 @@ int launch_channel_fmt(const GemmParams& p, int ta, int tb, int out_dt, hipStrea
 }
 
 }  // namespace
+
+void set_fp8_variant(int v) { g_fp8_variant = v; }
 
 // K-contiguous fp8 operands with every reduction range a multiple of the 128-deep slab.
 bool fast_fp8_supported(const GemmParams& p, bool block_scaled) {
@@ -463,7 +501,7 @@ int launch_fast_fp8_channel(const GemmParams& p, int ta, int tb, int out_dt, hip
 
 // sa must be laid out [ceil(K/128), m_total] (row-block major) for this kernel.
 int launch_fast_fp8_block(const GemmParams& p, hipStream_t s) {
-  return launch_fp8_cfg<Fp8Default, 0, 0, EPI_BLOCK, DT_BF16, false>(p, s);
+  return launch_fp8_cfg<0, 0, EPI_BLOCK, DT_BF16, false>(p, s);
 }
 
 }  // namespace tgg
