@@ -99,10 +99,12 @@ def test_tile_configurations_agree(dev, G, per_group, N, K):
         _native.set_option("variant", 0)
 
 
-@pytest.mark.parametrize("G,per_group,N,K", [(4, 128, 1024, 512), (8, 384, 1024, 256), (40, 256, 768, 384)])
+@pytest.mark.parametrize("G,per_group,N,K", [(4, 128, 1024, 512), (8, 384, 1024, 256), (40, 256, 768, 384), (128, 384, 768, 256),
+                                          (96, 1024, 512, 384)])
 def test_fp8_tile_configurations_agree(dev, G, per_group, N, K):
-    """The FP8 M-grouped kernels make the same choice between 256x128 and 256x256 tiles; either width gives the
-    same bits (block-scaled and per-channel), and the generic kernel agrees."""
+    """The FP8 M-grouped kernels choose on the device between 256x128 tiles, 256x256 tiles, and 256x256 tiles with
+    the path on which waves without rows sit a tile out (many half-empty tiles: the 128-group cases); forcing
+    either width gives the same bits (block-scaled and per-channel), and the generic kernel agrees."""
     from triton_grouped_gemm_amd.gemm.deep_gemm_ops import m_grouped_fp8_nt_contiguous
     from triton_grouped_gemm_amd.gemm.FP8.m_grouped_gemm_channel_expert import gmm_fp8_act_per_channel_w_per_expert
     from triton_grouped_gemm_amd.quant.fp8_cast import per_block_cast_to_fp8, per_token_cast_to_fp8

@@ -54,7 +54,9 @@ struct Fp8Cfg {
 
 // FA / FB: 0 = e4m3fn, 1 = e5m2 (the cbsz / blgp format codes of the f8f6f4 MFMA).
 // The whole kernel but for the group table, which the caller has built at byte SCHED_AT of the workgroup's LDS.
-template <class C, int FA, int FB, int EPI, int OUT, bool KGROUP, int SCHED_AT>
+// IDLE: waves whose block of a tile has no rows or columns sit that tile out (see the tile loop).  A separate
+// instantiation because the extra loop costs the plain one 1-1.5 % through register allocation alone.
+template <class C, int FA, int FB, int EPI, int OUT, bool KGROUP, int SCHED_AT, bool IDLE>
 TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   typedef Operand<C::BM, true> OpA;
   typedef Operand<C::BN, true> OpB;
@@ -131,14 +133,16 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   // Interleaved sweeps: with 1-byte operands an expert's weight panel set is twice as deep in K for the same
   // bytes, and letting all XCDs share the experts in flight through the memory-side cache measured ~3% faster
   // (and half the L2 fill traffic) than giving each XCD its own contiguous range of tiles.
-  const TileWalk walk = sched_walk(num_tiles, false);
+  // (tile ids are kept in 32 bits here: the tile space is far below 2^31 and scalar registers are scarce)
+  const TileWalk walk64 = sched_walk(num_tiles, false);
+  struct { int first, end, stride; } walk = {(int)walk64.first, (int)walk64.end, (int)walk64.stride};
   TileIo feed;
-  int64_t feed_id;
+  int feed_id;
   // The multiplying loop looks every tile up one tile ahead (it needs the tile's weight scales early); the feed
   // reaches that tile later and reuses the lookup instead of repeating its chain of dependent LDS reads.
   Tile nt;
-  int64_t nt_id = -1;
-  auto feed_seek = [&](int64_t id) {
+  int nt_id = -1;
+  auto feed_seek = [&](int id) {
     feed.kt_n = 0;
     feed.issued = 0;
     feed.a_base = feed.b_base = feed.s_base = (uint64_t)p.A;
@@ -247,7 +251,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
       for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
   };
 
-  for (int64_t tile_id = walk.first; tile_id < walk.end; tile_id += walk.stride) {
+  for (int tile_id = walk.first; tile_id < walk.end; tile_id += walk.stride) {
     const Tile cur = nt;
     const int kt_n = __builtin_amdgcn_readfirstlane(slabs_of(cur));
     float sbv = sbv_next;
@@ -255,6 +259,37 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
       nt = sched_tile<C::BM, C::BN>(p, sched, tile_id + walk.stride);
       nt_id = tile_id + walk.stride;
       sbv_next = load_sbv(nt);
+    }
+
+    // A wave whose block of the tile has no rows (groups of at most BM / WM rows) or no columns sits the tile
+    // out, as in gemm_fast.hip: it keeps its copies and the barriers going and reads the fragments the next tile
+    // starts with.
+    if (IDLE && !KGROUP && (wm0 >= cur.rows || cur.n0 + wn0 >= p.N)) {
+      for (int kt = 0; kt < kt_n; ++kt) {
+#pragma unroll
+        for (int k = C::TN; k < NC; ++k) {
+          copy_at(k);
+          __builtin_amdgcn_s_sleep(1);  // paced: the address unit's queue is shared with the working waves
+        }
+        const SlabCopy scn = begin_slab(ring & 1);
+        wait_vmcnt<0>();
+        if (BLOCK) asm volatile("" : "+v"(sbv_next));
+        __syncthreads();
+        sc = scn;
+#pragma unroll
+        for (int k = 0; k < C::TN; ++k) {
+          copy_at(k);
+          __builtin_amdgcn_s_sleep(1);
+        }
+        ++ring;
+      }
+      if (kt_n > 0) {
+        const char* sn = smem + (ring & 1) * C::STAGE_BYTES;
+#pragma unroll
+        for (int j = 0; j < C::TN; ++j) fb[j] = load_frag(sn + C::A_BYTES + (wn0 + 16 * j) * 128);
+        fa[0] = load_frag(sn + wm0 * 128);
+      }
+      continue;
     }
 
     // block scaling: the products that are still to be folded in when a slab ends (those of its last two
@@ -406,22 +441,35 @@ template <class C, int FA, int FB, int EPI, int OUT, bool KGROUP>
 __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   sched_init<C::BM>(p, *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::SCHED_OFF));
-  gemm_fp8_body<C, FA, FB, EPI, OUT, KGROUP, C::SCHED_OFF>(p);
+  gemm_fp8_body<C, FA, FB, EPI, OUT, KGROUP, C::SCHED_OFF, false>(p);
 }
 
-// Two tile widths in one kernel, chosen per launch on the device (see gemm_fast_auto_kernel in gemm_fast.hip): the
-// narrow tiles when all of them fit one round of the persistent workgroups, the wide ones otherwise.
+// Three bodies in one kernel, chosen per launch on the device from the group sizes (see gemm_fast_auto_kernel in
+// gemm_fast.hip): narrow tiles when all of them fit one round of the persistent workgroups; otherwise wide tiles,
+// with the sit-out path when at least one tile in eight is at most half full (groups whose size modulo 256 lies
+// in 1..128: decode-sized groups), without it otherwise.
 template <class CW, class CN, int FA, int FB, int EPI, int OUT>
 __global__ __launch_bounds__(CW::THREADS) void gemm_fp8_auto_kernel(const GemmParams p) {
   static_assert(CW::BM == CN::BM && CW::THREADS == CN::THREADS, "one group table, one launch shape");
   static_assert(CN::SMEM_BYTES <= CW::SCHED_OFF, "the narrow configuration must not reach the shared group table");
+  static_assert(CW::THREADS >= kFastMaxGroups && CW::BM == 256, "one group per thread in the count below");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + CW::SCHED_OFF);
   sched_init<CW::BM>(p, sched);
-  if (__builtin_expect(sched_num_tiles<CN::BM, CN::BN>(p, sched) > (int64_t)gridDim.x, 1))
-    gemm_fp8_body<CW, FA, FB, EPI, OUT, false, CW::SCHED_OFF>(p);
+  int half_full = 0;
+  if ((int)threadIdx.x < p.G) {
+    const int r = sched.rows[threadIdx.x] & 255;
+    half_full = r >= 1 && r <= 128;
+  }
+  const int n_half_full = __syncthreads_count(half_full);
+  const bool narrow = sched_num_tiles<CN::BM, CN::BN>(p, sched) <= (int64_t)gridDim.x;
+  const bool sit_out = n_half_full * 8 >= sched.tile0[p.G];
+  if (__builtin_expect(!narrow && !sit_out, 1))  // marked likely: the register allocator then favours this body's loops
+    gemm_fp8_body<CW, FA, FB, EPI, OUT, false, CW::SCHED_OFF, false>(p);
+  else if (narrow)
+    gemm_fp8_body<CN, FA, FB, EPI, OUT, false, CW::SCHED_OFF, true>(p);
   else
-    gemm_fp8_body<CN, FA, FB, EPI, OUT, false, CW::SCHED_OFF>(p);
+    gemm_fp8_body<CW, FA, FB, EPI, OUT, false, CW::SCHED_OFF, true>(p);
 }
 
 template <class Kern>
