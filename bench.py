@@ -29,14 +29,14 @@ PEAK_HBM_GBS = 8000.0
 # plain 1 GiB device copy: x2.0 and x1.0).  The runs and their figures are listed in profiles/hbm_traffic.txt.
 # FETCH_SIZE includes L2 fills served by the memory-side cache, so these are upper bounds on DRAM traffic.
 MEASURED_TRAFFIC_GB = {
-    "bf16_m_grouped_gateup_nt": 11.81,
-    "bf16_m_grouped_gateup_nn": 11.45,
-    "bf16_m_grouped_gateup_fp8_out": 10.74,
-    "bf16_m_grouped_down_nt": 5.47,
-    "bf16_m_grouped_down_nn": 5.46,
-    "bf16_masked_decode": 2.59,
-    "bf16_k_grouped_wgrad": 32.02,
-    "fp8_block_m_grouped": 20.88,
+    "bf16_m_grouped_gateup_nt": 11.82,
+    "bf16_m_grouped_gateup_nn": 11.50,
+    "bf16_m_grouped_gateup_fp8_out": 10.47,
+    "bf16_m_grouped_down_nt": 5.51,
+    "bf16_m_grouped_down_nn": 5.45,
+    "bf16_masked_decode": 2.60,
+    "bf16_k_grouped_wgrad": 34.13,
+    "fp8_block_m_grouped": 18.66,
     "quant_trans128": 8.12,
     "moe_permute": 3.06,      # the row mover (the sort kernels move < 1 % of that)
     "moe_unpermute": 3.07,
