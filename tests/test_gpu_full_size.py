@@ -155,7 +155,7 @@ def test_config5_fp8_block_scaled_full_size(dev):
         o = out[s0:s0 + n].float()
         worst = max(worst, ((o - ref).abs().max() / max(o.abs().max(), ref.abs().max())).item())
     assert worst <= 2e-2, worst
-    assert worst <= 2.0 ** -7, worst  # only the bf16 output rounding remains
+    assert worst <= 2.0 ** -7, worst  # the bf16 output rounding dominates (the MFMA's own truncation is ~2^-13)
     # CPU oracle on one sampled block
     g = _sample_groups(sizes_cpu)[1]
     s0, n = starts[g], min(int(sizes_cpu[g]), 128)
