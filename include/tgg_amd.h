@@ -154,7 +154,7 @@ int tgg_debug_tile_order(const int64_t* sizes, int G, int mode, int64_t m_total,
  *   "variant"       int  tile configuration of the tuned kernels (16-bit, and FP8 M-grouped): 0 (default) = chosen per launch on the
  *                        device from the group sizes -- 256x128 when all such tiles fit one round of the persistent
  *                        workgroups, 256x256 otherwise; 1 = always 256x128; 2 = always 256x256
- *   "tile_split"    0/1  16-bit M-grouped: per-XCD contiguous tile ranges (default 1) or interleaved sweeps
+ *   "tile_split"    0/1  M-grouped tuned kernels: per-XCD contiguous tile ranges (default 1) or interleaved sweeps
  *   "n_chunk"       int  column tiles per chunk of the tile order (0 = automatic, at most eight)
  *   "store_nt"      0/1  write the output with non-temporal stores (default 1) */
 int tgg_set_option(const char* key, int value);

@@ -130,11 +130,9 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   };
 
   // The copy stream (see gemm_fast.hip): slab q of the workgroup's whole slab sequence lives in buffer q % 2.
-  // Interleaved sweeps: with 1-byte operands an expert's weight panel set is twice as deep in K for the same
-  // bytes, and letting all XCDs share the experts in flight through the memory-side cache measured ~3% faster
-  // (and half the L2 fill traffic) than giving each XCD its own contiguous range of tiles.
-  // (tile ids are kept in 32 bits here: the tile space is far below 2^31 and scalar registers are scarce)
-  const TileWalk walk64 = sched_walk(num_tiles, false);
+  // M-grouped: every XCD owns a contiguous range of tiles, as in the 16-bit kernels (measured +2 % over
+  // interleaved sweeps); K-grouped: interleaved, since a tile's cost follows its group's token count.
+  const TileWalk walk64 = sched_walk(num_tiles, !KGROUP && p.tile_split);
   struct { int first, end, stride; } walk = {(int)walk64.first, (int)walk64.end, (int)walk64.stride};
   TileIo feed;
   int feed_id;
