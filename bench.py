@@ -29,14 +29,16 @@ PEAK_HBM_GBS = 8000.0
 # plain 1 GiB device copy: x2.0 and x1.0).  The runs and their figures are listed in profiles/hbm_traffic.txt.
 # FETCH_SIZE includes L2 fills served by the memory-side cache, so these are upper bounds on DRAM traffic.
 MEASURED_TRAFFIC_GB = {
-    "bf16_m_grouped_gateup_nt": 11.82,
-    "bf16_m_grouped_gateup_nn": 11.50,
-    "bf16_m_grouped_gateup_fp8_out": 10.47,
-    "bf16_m_grouped_down_nt": 5.51,
-    "bf16_m_grouped_down_nn": 5.45,
-    "bf16_masked_decode": 2.60,
-    "bf16_k_grouped_wgrad": 34.13,
-    "fp8_block_m_grouped": 18.66,
+    "bf16_m_grouped_gateup_nt": 11.80,
+    "bf16_m_grouped_gateup_nn": 11.38,
+    "bf16_m_grouped_gateup_fp8_out": 10.56,
+    "bf16_m_grouped_down_nt": 5.48,
+    "bf16_m_grouped_down_nn": 5.43,
+    "bf16_masked_decode": 2.59,
+    "bf16_k_grouped_wgrad": 31.56,
+    "fp8_block_m_grouped": 21.69,
+    "fp8_channel_m_grouped": 26.42,
+    "fp8_channel_k_grouped": 18.40,
     "quant_trans128": 8.12,
     "moe_permute": 3.06,      # the row mover (the sort kernels move < 1 % of that)
     "moe_unpermute": 3.07,
@@ -53,6 +55,8 @@ WORKLOADS = {
     "bf16_masked_decode": ("masked", 4096, 1536, True),
     "bf16_k_grouped_wgrad": ("kg", 4096, 3072, False),      # N_DIM, M_DIM
     "fp8_block_m_grouped": ("fp8", 3072, 4096, True),
+    "fp8_channel_m_grouped": ("fp8c", 3072, 4096, True),     # per-token x per-channel scales, same shape
+    "fp8_channel_k_grouped": ("fp8ck", 4096, 3072, False),   # N_DIM, M_DIM; tokens along K
     "quant_trans128": ("quant", 4096, 0, False),
     # MoE token movement either side of the GEMMs: 81920 tokens x top-8 = 655360 rows of 2048 bf16
     "moe_permute": ("permute", 2048, 8, False),       # hidden, topK
@@ -163,6 +167,30 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
         nbytes = M_TOTAL * K + 4.0 * M_TOTAL * K / 128 + G * N * K + 4.0 * G * (N / 128) * (K / 128) + 2.0 * M_TOTAL * N
         return (fn, 2.0 * M_TOTAL * N * K, nbytes, "fp8",
                 dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, recipe="1x128 act / 128x128 weight, e4m3fn", seed=seed), None)
+    if kind == "fp8c":
+        from triton_grouped_gemm_amd.gemm.FP8.m_grouped_gemm_channel_expert import gmm_fp8_act_per_channel_w_per_expert
+        gen = torch.Generator(device=dev).manual_seed(seed + 3)
+        a = wl.randn_bf16((M_TOTAL, K), 1.0, seed + 1, dev).to(torch.float8_e4m3fn)
+        w = wl.randn_bf16((G, N, K), 1.0, seed + 2, dev).to(torch.float8_e4m3fn)
+        sa = torch.rand(M_TOTAL, 1, device=dev, generator=gen) + 0.5
+        sb = torch.rand(G * N, device=dev, generator=gen) + 0.5
+        fn = lambda: gmm_fp8_act_per_channel_w_per_expert(a, sa, w, sb, sizes, torch.bfloat16)
+        nbytes = M_TOTAL * K + 4.0 * M_TOTAL + G * N * K + 4.0 * G * N + 2.0 * M_TOTAL * N
+        return (fn, 2.0 * M_TOTAL * N * K, nbytes, "fp8",
+                dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, recipe="per-token x per-channel scales, e4m3fn", seed=seed), None)
+    if kind == "fp8ck":
+        from triton_grouped_gemm_amd.gemm.FP8.k_grouped_gemm_channel_expert import matmul as k_grouped_fp8
+        m_dim, n_dim = K, N
+        gen = torch.Generator(device=dev).manual_seed(seed + 3)
+        x = wl.randn_bf16((m_dim, M_TOTAL), 1.0, seed + 1, dev).to(torch.float8_e4m3fn)
+        y = wl.randn_bf16((n_dim, M_TOTAL), 1.0, seed + 2, dev).to(torch.float8_e4m3fn)
+        xs = torch.rand(m_dim, G, device=dev, generator=gen) + 0.5
+        ys = torch.rand(n_dim, G, device=dev, generator=gen) + 0.5
+        fn = lambda: k_grouped_fp8(x, xs, y, ys, sizes, m_dim, n_dim, M_TOTAL, G)
+        nbytes = 1.0 * M_TOTAL * (m_dim + n_dim) + 4.0 * G * (m_dim + n_dim) + 2.0 * G * m_dim * n_dim
+        return (fn, 2.0 * M_TOTAL * m_dim * n_dim, nbytes, "fp8",
+                dict(workload=name, G=G, M=m_dim, N=n_dim, K_total=M_TOTAL, recipe="per-channel x per-expert scales, e4m3fn",
+                     seed=seed), None)
     if kind == "quant":
         from triton_grouped_gemm_amd.quant.trans_per_block_quant_expand_128x import trans_per_block_quant_expand_128x
         x = wl.randn_bf16((M_TOTAL, N), 1.0, seed + 1, dev)
