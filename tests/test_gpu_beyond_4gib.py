@@ -180,3 +180,51 @@ def test_permute_unpermute_beyond_4gib(dev):
     del un
     quarter = torch.full((T, topk), 0.25, device=dev)
     assert torch.equal(ops.unpermute(perm, rmap, quarter), x)  # four exact quarters of one bf16 value sum exactly
+
+
+def test_fp8_channel_operands_beyond_4gib(dev):
+    """Per-channel FP8, M-grouped (A of 4.7 GB) and K-grouped (x of 4.7 GB, tokens along K): rows on both sides of
+    byte 2^32 against torch's fp32 matmul; the bound allows for the matrix instruction's product truncation."""
+    from triton_grouped_gemm_amd.gemm.FP8.k_grouped_gemm_channel_expert import matmul as k_grouped_fp8
+    from triton_grouped_gemm_amd.gemm.FP8.m_grouped_gemm_channel_expert import gmm_fp8_act_per_channel_w_per_expert
+
+    def close(out, ref, mag):
+        err = (out.float() - ref).abs()
+        return bool((err <= ref.abs() * (2.0 ** -8 * 1.05) + 2.0 ** -12 * mag + 1e-30).all())
+
+    gen = torch.Generator(device=dev).manual_seed(311)
+    M, N, K = sum(SIZES), 256, 4096
+    a = workloads.randn_bf16((M, K), 1.0, 312, dev).to(torch.float8_e4m3fn)
+    assert a.numel() > 1 << 32
+    w = workloads.randn_bf16((len(SIZES), N, K), 1.0, 313, dev).to(torch.float8_e4m3fn)
+    sa = torch.rand(M, 1, device=dev, generator=gen) + 0.5
+    sb = torch.rand(len(SIZES) * N, device=dev, generator=gen) + 0.5
+    out = gmm_fp8_act_per_channel_w_per_expert(a, sa, w, sb, torch.tensor(SIZES, dtype=torch.int32, device=dev), torch.bfloat16)
+    for lo, hi in BLOCKS:
+        for r0 in range(lo, hi, 100):
+            g = _group_of(r0, SIZES)
+            r1 = min(r0 + 100, hi, sum(SIZES[:g + 1]))
+            scale = sa[r0:r1] * sb[g * N:(g + 1) * N][None, :]
+            ref = (a[r0:r1].float() @ w[g].float().t()) * scale
+            mag = (a[r0:r1].float().abs() @ w[g].float().abs().t()) * scale
+            assert close(out[r0:r1], ref, mag), (r0, r1)
+    del a, w, out
+    # K-grouped: x [Md, Ktot], y [Nd, Ktot]; row r of x starts at byte r * Ktot, so rows from 2^32 / Ktot on lie beyond
+    tokens = [128 * n for n in (3000, 0, 9000, 1, 5187)]
+    Ktot, Md, Nd, G = sum(tokens), 2048, 256, len(tokens)
+    assert Md * Ktot > 1 << 32
+    x = workloads.randn_bf16((Md, Ktot), 1.0, 314, dev).to(torch.float8_e4m3fn)
+    y = workloads.randn_bf16((Nd, Ktot), 1.0, 315, dev).to(torch.float8_e4m3fn)
+    xs = torch.rand(Md, G, device=dev, generator=gen) + 0.5
+    ys = torch.rand(Nd, G, device=dev, generator=gen) + 0.5
+    out = k_grouped_fp8(x, xs, y, ys, torch.tensor(tokens, dtype=torch.int32, device=dev), Md, Nd, Ktot, G)
+    assert out.shape == (G, Md, Nd) and torch.count_nonzero(out[1]) == 0
+    row_mark = (1 << 32) // Ktot
+    rows = torch.cat([torch.arange(0, 64), torch.arange(row_mark - 64, row_mark + 64), torch.arange(Md - 64, Md)]).to(dev)
+    start = 0
+    for g, n in enumerate(tokens):
+        if n:
+            xg, yg = x[rows, start:start + n].float(), y[:, start:start + n].float()
+            scale = xs[rows, g][:, None] * ys[:, g][None, :]
+            assert close(out[g][rows], (xg @ yg.t()) * scale, (xg.abs() @ yg.abs().t()) * scale), f"group {g}"
+        start += n
