@@ -199,3 +199,20 @@ def test_fp8_random_shapes(dev, seed):
                         f"seed {seed} case {case} block G={G} N={N} K={K} g={g}"
                 assert bool((out[start + n:start + pn] == 9.0).all()), f"seed {seed} case {case}: pad rows written"
                 start += pn
+
+
+@pytest.mark.parametrize("num_cu", [1, 7, 100, 128, 1000])
+def test_any_number_of_workgroups_gives_the_same_bits(dev, num_cu):
+    """``numSM`` limits the persistent grid (1 workgroup, counts that are not multiples of the eight XCDs, more
+    than the chip has): the tile walk changes, the device-side tile-width choice may change, the bits do not."""
+    rng = random.Random(77)
+    sizes = [rng.choice([0, 3, 128, 200, 256, 300, 700]) for _ in range(24)]
+    st = torch.tensor(sizes, dtype=torch.int32, device=dev)
+    torch.manual_seed(77)
+    a = (torch.randn(sum(sizes), 264, device=dev) * 264 ** -0.5).to(torch.bfloat16)
+    b = torch.randn(24, 392, 264, device=dev).to(torch.bfloat16)
+    ak = torch.randn(sum(sizes), 520, device=dev).to(torch.bfloat16)
+    bk = torch.randn(sum(sizes), 392, device=dev).to(torch.bfloat16)
+    assert torch.equal(m_grouped_gemm(a, b, st, True, num_cu), m_grouped_gemm(a, b, st, True))
+    assert torch.equal(m_grouped_gemm(a, b.transpose(1, 2).contiguous(), st, False, num_cu), m_grouped_gemm(a, b, st, True))
+    assert torch.equal(k_grouped_gemm(ak, bk, st, numSM=num_cu), k_grouped_gemm(ak, bk, st))
