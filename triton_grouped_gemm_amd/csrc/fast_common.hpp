@@ -15,6 +15,9 @@ template <int N> TGG_DEV void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
+// All of this wave's vector-memory traffic and all of its LDS reads have completed.
+TGG_DEV void wait_vmcnt0_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(7 << 4); }
+
 // One wave-wide 16-byte-per-lane copy global -> LDS.  The LDS destination is m0 + lane * 16, the
 // global source is the descriptor base + voff (bounds-checked: out-of-range lanes write zeros).
 // Written as inline assembly on purpose: the compiler does not model the copy, so it cannot

@@ -314,7 +314,9 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
         if (i < C::TM - 1) {
           fa[(i + 1) & 1] = load_frag(sa + (wm0 + 16 * (i + 1)) * 128);
         } else {
-          wait_vmcnt<0>();
+          // this wave's share of the next slab has landed, and its reads of the current slab (the last A
+          // fragment was requested a row block ago) are complete: after the barrier the buffer is overwritten
+          wait_vmcnt0_lgkmcnt0();
           if (BLOCK) asm volatile("" : "+v"(sbv_next));  // nothing of this wave is in flight: touching it costs no wait
           __syncthreads();
           sc = scn;
