@@ -216,3 +216,26 @@ def test_any_number_of_workgroups_gives_the_same_bits(dev, num_cu):
     assert torch.equal(m_grouped_gemm(a, b, st, True, num_cu), m_grouped_gemm(a, b, st, True))
     assert torch.equal(m_grouped_gemm(a, b.transpose(1, 2).contiguous(), st, False, num_cu), m_grouped_gemm(a, b, st, True))
     assert torch.equal(k_grouped_gemm(ak, bk, st, numSM=num_cu), k_grouped_gemm(ak, bk, st))
+
+
+def test_non_finite_inputs_stay_in_their_row_and_column(dev):
+    """A NaN or an infinity in one activation row (or one weight column) shows up in that output row (column) only,
+    as in torch's matmul: nothing leaks through shared tiles, staging or the transposing epilogue."""
+    sizes = [300, 0, 129, 700]
+    st = torch.tensor(sizes, dtype=torch.int32, device=dev)
+    torch.manual_seed(5)
+    M, N, K = sum(sizes), 520, 264
+    a = (torch.randn(M, K, device=dev) * K ** -0.5).to(torch.bfloat16)
+    b = torch.randn(len(sizes), N, K, device=dev).to(torch.bfloat16)
+    clean = m_grouped_gemm(a, b, st, True)
+    a2, b2 = a.clone(), b.clone()
+    a2[17, 3] = float("nan")          # group 0
+    a2[301, 200] = float("inf")       # group 2, second row
+    b2[3, 77, 5] = float("nan")       # group 3, column 77
+    out = m_grouped_gemm(a2, b2, st, True)
+    expect_bad = torch.zeros(M, N, dtype=torch.bool, device=dev)
+    expect_bad[17] = True
+    expect_bad[301] = True
+    expect_bad[429:, 77] = True       # group 3 holds rows 429..1128
+    assert bool((~torch.isfinite(out.float()) == expect_bad).all())
+    assert torch.equal(out[~expect_bad], clean[~expect_bad])
