@@ -86,3 +86,24 @@ def test_sizes_from_explicit_layouts():
         assert sizes_from_layout(rows, len(sizes), block_m, False).tolist() == sizes
         assert sizes_from_layout(ends, len(sizes), block_m, True).tolist() == sizes
         assert sizes_from_layout(rows.to(torch.int64), len(sizes), block_m, False).dtype == torch.int32
+
+
+def test_reference_named_helpers():
+    """gemm/BF16/utils.py of the reference: the per-group torch loop, the group-size draw and the two checks."""
+    import random
+
+    import torch
+
+    from triton_grouped_gemm_amd.gemm.BF16.utils import allclose, generate_random_list, gmm, row_max_normalization
+    random.seed(3)
+    for length, total in [(8, 1000), (1, 17), (128, 655360), (5, 4)]:
+        sizes = generate_random_list(length, total)
+        assert len(sizes) == length and sum(sizes) == total and min(sizes[:-1] + [0]) >= 0
+    sizes = [3, 0, 5]
+    a, b = torch.randn(8, 6), torch.randn(3, 6, 4)
+    out = gmm(a, b, torch.tensor(sizes))
+    assert out.shape == (8, 4)
+    assert torch.equal(out[:3], a[:3] @ b[0]) and torch.equal(out[3:], a[3:] @ b[2])
+    assert torch.equal(gmm(a, b.transpose(1, 2).contiguous(), torch.tensor(sizes), trans_b=True), out)
+    assert allclose(out, out) and not allclose(out, out + 1.0)
+    assert float(row_max_normalization(a).abs().max(dim=-1).values.max()) <= 1.0
