@@ -83,12 +83,15 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   const int kblocks = (p.K + 127) >> 7;
   const int nblocks = (p.N + 127) >> 7;
 
-  // A fragment of the 16x16x128 multiply is 32 consecutive K values per lane: K = 32 lg + (0..31) of row or
-  // column (block + l16), i.e. chunks 2 lg and 2 lg + 1 of its 128-byte LDS row.
+  // A fragment of the 16x16x128 multiply is 32 K values per lane.  Which 32 is free as long as both operands
+  // agree (a dot product does not care about the order of its terms): lane group lg takes 16-byte chunks lg and
+  // lg + 4 of the row's 128 bytes, so that each of the two reads has the lanes of a wave on four neighbouring
+  // chunks, the access pattern of the 16-bit kernels.  Chunks 2 lg and 2 lg + 1 (the instruction's nominal K
+  // order) collide in the LDS banks: 3.2 conflict cycles per read and 1.6 % slower overall.
   const int fsw = (l16 / 2) % 8;
   int rd[2];
 #pragma unroll
-  for (int h = 0; h < 2; ++h) rd[h] = l16 * 128 + (((2 * lg + h) ^ fsw) << 4);
+  for (int h = 0; h < 2; ++h) rd[h] = l16 * 128 + (((lg + 4 * h) ^ fsw) << 4);
   // the fragment of the 16-row block starting at LDS address q
   auto load_frag = [&](const char* q) -> i32x8_t {
     const i32x4_t lo = *(const i32x4_t*)(q + rd[0]);
