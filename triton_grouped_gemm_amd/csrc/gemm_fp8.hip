@@ -344,7 +344,10 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
             fb[j] = load_frag(sn + C::A_BYTES + (wn0 + 16 * j) * 128);
           } else {
             if (n == C::TN * (C::TM - 2) + 1) scn = begin_slab(ring & 1);  // scalar work under a multiply
-            copy_at(C::TN + n);
+            // block-scaled: one copy per multiply; per-channel (no folds between the multiplies, so the copies of
+            // all waves come closer together and crowd the address unit's queue): one per two multiplies, +0.9 %
+            if (BLOCK) copy_at(C::TN + n);
+            else if (n % 2 == 0) copy_at(C::TN + n / 2);
           }
           if (BLOCK && jj == 0) srow[i] *= sb_cur;
           if (BLOCK) {
