@@ -53,3 +53,60 @@ def test_forward_and_weight_gradient_in_one_graph(dev):
         ref = m_grouped_gemm(a, b, sizes, True)
         assert torch.equal(out, ref), f"replay {it}"
         assert torch.equal(dw, k_grouped_gemm(g, a, sizes)), f"replay {it} (weight gradient)"
+
+
+def test_group_sizes_may_change_between_replays(dev):
+    """Group sizes are read on the device, so one captured graph serves any routing: between replays the sizes
+    buffer is rewritten so that the kernels' device-side choices change (few narrow tiles; many half-empty tiles;
+    large groups), for the 16-bit and the block-scaled FP8 M-grouped GEMM."""
+    from triton_grouped_gemm_amd.quant.fp8_cast import per_block_cast_to_fp8, per_token_cast_to_fp8
+    G, M, N, K = 64, 64 * 256, 1024, 512
+    a, b = _randn((M, K), 21, dev), _randn((G, N, K), 22, dev)
+    aq, sa = per_token_cast_to_fp8(a, scales_mn_major=True)
+    wq, sb = per_block_cast_to_fp8(b)
+    sizes = torch.zeros(G, dtype=torch.int32, device=dev)
+    out16 = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    out8 = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+
+    def step():
+        st = _native.stream_of(a)
+        _native.call("tgg_m_grouped_gemm", a.data_ptr(), b.data_ptr(), out16.data_ptr(), sizes.data_ptr(), 0, G, M, N, K, 1,
+                     _native.DTYPE_CODE[torch.bfloat16], -1, st)
+        _native.call("tgg_m_grouped_gemm_fp8_block", aq.data_ptr(), sa.data_ptr(), wq.data_ptr(), sb.data_ptr(),
+                     out8.data_ptr(), sizes.data_ptr(), 0, G, M, N, K, 128, 1, -1, st)
+
+    routings = [
+        [128] * 3 + [0] * (G - 3),                 # 3 row tiles x 8 narrow column tiles: the narrow configuration
+        [128] * G,                                  # every tile half empty: waves sit tiles out
+        [256] * G,                                  # full tiles
+        [1024, 0, 384] + [128] * 8 + [0] * (G - 11),
+    ]
+    sizes.copy_(torch.tensor(routings[0], dtype=torch.int32))
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for it, routing in enumerate(routings * 2):
+        sizes.copy_(torch.tensor(routing, dtype=torch.int32))
+        out16.fill_(7.0)
+        out8.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        rows = sum(routing)
+        ref16 = m_grouped_gemm(a, b, sizes, True)
+        ref8 = torch.full_like(out8, 7.0)  # the same call, eagerly (the wrapper insists on M = sum of the padded sizes)
+        _native.call("tgg_m_grouped_gemm_fp8_block", aq.data_ptr(), sa.data_ptr(), wq.data_ptr(), sb.data_ptr(),
+                     ref8.data_ptr(), sizes.data_ptr(), 0, G, M, N, K, 128, 1, -1, _native.stream_of(a))
+        assert torch.equal(out16[:rows], ref16[:rows]), f"replay {it}"
+        placed = 0
+        for n in routing:  # block-scaled layout: every group starts at a multiple of 128 rows
+            assert torch.equal(out8[placed:placed + n], ref8[placed:placed + n]), f"replay {it} (fp8)"
+            placed += (n + 127) // 128 * 128
+        n0 = routing[0]
+        ad = aq[:n0].float() * sa[:n0].repeat_interleave(128, dim=1)
+        wd = wq[0].float() * sb[0].repeat_interleave(128, dim=0).repeat_interleave(128, dim=1)
+        exact = ad @ wd.t()
+        assert float((out8[:n0].float() - exact).abs().max()) <= 2.0 ** -7 * float(exact.abs().max()), f"replay {it} (fp8 values)"
+        assert bool((out16[rows:] == 7.0).all()) and bool((out8[placed:] == 7.0).all()), f"replay {it}: rows past the groups"
