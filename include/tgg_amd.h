@@ -149,6 +149,14 @@ int tgg_moe_unpermute_bwd(const void* grad_output, const void* fwd_input, const 
 int tgg_debug_tile_order(const int64_t* sizes, int G, int mode, int64_t m_total, int64_t aux, int N, int tile,
                          int grid, int split, int64_t* out, int64_t capacity, int64_t* num_tiles);
 
+/* Test hook, host only: the group table's row-tile lookup that the transposing quantizer and the GEMM schedulers share.
+ * Row tile i (counted over the groups' ceil(size / tile) tiles in group order, as m_indices_pad does,
+ * gemm/BF16/m_grouped_gemm_TMA.py:297-326; the quantizer's token_start / pad_start arithmetic,
+ * quant/trans_per_block_quant_expand_128x.py:91-110) -> out[i] = {group, first row in A, valid rows}.
+ * modes as in tgg_debug_tile_order (0, 1, 2); n_chunk is the tile-order option, which must not change the answer. */
+int tgg_debug_row_tiles(const int64_t* sizes, int G, int mode, int64_t m_total, int64_t aux, int tile, int n_chunk,
+                        int64_t* out, int64_t capacity, int64_t* num_row_tiles);
+
 /* Library controls (process-wide, meant for tests and tuning; returns 1 for an unknown key):
  *   "force_generic" 0/1  route every GEMM through the shape-agnostic kernel
  *   "variant"       int  tile configuration of the tuned kernels (16-bit, and FP8 M-grouped): 0 (default) = chosen per launch on the

@@ -56,6 +56,52 @@ def test_trans_quant_bit_exact(dev, dtype, sizes, N):
     assert np.array_equal(codes_np(codes), rc)
 
 
+def _check_trans_quant(dev, x, sizes, dtype=torch.float8_e4m3fn, size_dtype=torch.int32):
+    codes, scales, padded = trans_per_block_quant_expand_128x(
+        x.to(dev), torch.tensor(sizes, dtype=size_dtype, device=dev), dtype=dtype)
+    rc, rs, rp = quant_ref.trans_per_block_quant_expand_128x(to_np_f32(x), sizes, FMT[dtype])
+    assert tuple(codes.shape) == rc.shape and tuple(scales.shape) == rs.shape
+    assert padded.tolist() == rp.tolist()
+    assert np.array_equal(scales.cpu().numpy().view(np.uint32), rs.view(np.uint32))
+    assert np.array_equal(codes_np(codes), rc)
+
+
+@pytest.mark.parametrize("N", [1152, 2048, 4096, 7168])
+def test_trans_quant_bit_exact_wide(dev, N):
+    """More than eight 128-column blocks per row (the GEMM tile order cuts such widths into column chunks; the
+    quantizer must not follow it), ragged groups of three and more row blocks, an empty group."""
+    sizes = [300, 0, 417, 128, 385, 1]
+    x = _randn((sum(sizes), N), 90 + N % 7, 1.5)
+    _check_trans_quant(dev, x, sizes)
+
+
+def test_trans_quant_bit_exact_wide_many_groups(dev):
+    """G > 256 (the large group table) at N = 2048, int64 sizes, e5m2."""
+    sizes = [(i * 53) % 290 for i in range(300)]
+    x = _randn((sum(sizes), 2048), 91)
+    _check_trans_quant(dev, x, sizes, torch.float8_e5m2, torch.int64)
+
+
+@pytest.mark.parametrize("n_chunk", [1, 2])
+def test_trans_quant_ignores_gemm_tile_order_option(dev, n_chunk):
+    """The column-chunk option of the GEMM tile order must not reach the quantizer."""
+    sizes = [300, 0, 130, 128]
+    x = _randn((sum(sizes), 512), 92)
+    _native.set_option("n_chunk", n_chunk)
+    try:
+        _check_trans_quant(dev, x, sizes)
+    finally:
+        _native.set_option("n_chunk", 0)
+
+
+def test_trans_quant_reference_self_test_shape(dev):
+    """The shape of the reference's own self-test: 65536 x 7168 bf16, 32 groups of 2048 rows
+    (quant/trans_per_block_quant_expand_128x.py:276-277), every block against the oracle."""
+    sizes = [2048] * 32
+    x = _randn((65536, 7168), 93)
+    _check_trans_quant(dev, x, sizes)
+
+
 def test_trans_quant_special_values(dev):
     """All-zero blocks (scale clamps to 1e-12, codes 0), huge and tiny magnitudes, exact ties."""
     sizes = [128, 128, 128]

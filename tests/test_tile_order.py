@@ -106,3 +106,42 @@ def test_runs_of_an_xcd_are_near_square():
         assert len(mine) == 32
         assert len(set(mine[:, 3].tolist())) * len(set(mine[:, 5].tolist())) == 32  # a full rectangle
         assert len(set(mine[:, 3].tolist())) + len(set(mine[:, 5].tolist())) <= 12   # 4 x 8
+
+
+def row_tiles(sizes, mode, m_total, aux, tile, n_chunk=0):
+    lib = _native.load()
+    s = np.asarray(sizes, dtype=np.int64)
+    cap = 1 << 14
+    out = np.zeros((cap, 3), dtype=np.int64)
+    n = ctypes.c_int64(0)
+    rc = lib.tgg_debug_row_tiles(s.ctypes.data, len(s), mode, m_total, aux, tile, n_chunk, out.ctypes.data, cap,
+                                 ctypes.byref(n))
+    assert rc == 0, lib.tgg_last_error().decode()
+    return out[:n.value].tolist()
+
+
+@pytest.mark.parametrize("tile", [128, 256])
+@pytest.mark.parametrize("n_chunk", [0, 1, 2, 8])
+@pytest.mark.parametrize("sizes", [
+    [300, 0, 130, 128],          # the case on which the transposing quantizer once read the wrong row block
+    [1, 0, 127, 129, 256, 3, 0, 300],
+    [2048] * 32,
+    [0, 0, 5],
+    list(range(0, 700, 37)),
+])
+def test_row_tile_lookup(tile, n_chunk, sizes):
+    """The lookup the transposing quantizer uses (global row tile -> group, first row, valid rows) against a plain
+    Python enumeration of the groups' tiles; it must not depend on the column-chunk option of the GEMM tile order."""
+    exp, start = [], 0
+    for g, sz in enumerate(sizes):
+        for mt in range(-(-sz // tile)):
+            exp.append([g, start + mt * tile, min(tile, sz - mt * tile)])
+        start += sz
+    assert row_tiles(sizes, MG, sum(sizes), 0, tile, n_chunk) == exp
+
+
+def test_row_tile_lookup_padded_and_masked():
+    sizes = [100, 0, 130, 128]
+    assert row_tiles(sizes, MG_PAD, 512, 128, 128) == [[0, 0, 100], [2, 128, 128], [2, 256, 2], [3, 384, 128]]
+    assert row_tiles([512, 0, 77, 300], MASKED, 2048, 512, 256) == [
+        [0, 0, 256], [0, 256, 256], [2, 1024, 77], [3, 1536, 256], [3, 1792, 44]]

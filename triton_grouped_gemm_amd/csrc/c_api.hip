@@ -401,6 +401,45 @@ int tgg_debug_tile_order(const int64_t* sizes, int G, int mode, int64_t m_total,
   return set_error("tile must be 256 (tuned kernels) or 128 (shape-agnostic kernel)");
 }
 
+int tgg_debug_row_tiles(const int64_t* sizes, int G, int mode, int64_t m_total, int64_t aux, int tile, int n_chunk,
+                        int64_t* out, int64_t capacity, int64_t* num_row_tiles) {
+  if (!sizes || !out || !num_row_tiles) return set_error("null pointer");
+  if (G < 1 || G > TGG_MAX_GROUPS) return set_error("G=%d outside [1, %d]", G, TGG_MAX_GROUPS);
+  if (m_total < 0) return set_error("bad m_total");
+  if (mode != MODE_MG && mode != MODE_MG_PAD && mode != MODE_MASKED)
+    return set_error("mode %d not supported by the row-tile hook", mode);
+  if (tile != 128 && tile != 256) return set_error("tile must be 128 or 256");
+  GemmParams p = zero_params();
+  p.sizes = sizes;
+  p.sizes_i64 = 1;
+  p.G = G;
+  p.mode = mode;
+  p.m_total = m_total;
+  p.N = 128;
+  p.n_chunk = n_chunk;  // must not influence the row-tile lookup
+  p.align = mode == MODE_MG_PAD ? (int)aux : 1;
+  p.m_stride = mode == MODE_MASKED ? aux : 0;
+  if (mode == MODE_MG_PAD && p.align < 1) return set_error("alignment must be positive");
+  SchedTable* t = new SchedTable;
+  for (int g = 0; g < G; ++g) sched_load_group(p, *t, g);
+  if (tile == 128) sched_prefix<128>(p, *t); else sched_prefix<256>(p, *t);
+  const int total = t->tile0[G];
+  *num_row_tiles = total;
+  int g_prev = -1;
+  for (int mt = 0; mt < total; ++mt) {
+    const RowTile a = tile == 128 ? sched_row_tile<128>(*t, G, mt) : sched_row_tile<256>(*t, G, mt);
+    const RowTile h = tile == 128 ? sched_row_tile<128>(*t, G, mt, g_prev) : sched_row_tile<256>(*t, G, mt, g_prev);
+    if (a.g != h.g || a.row0 != h.row0 || a.rows != h.rows) {
+      delete t;
+      return set_error("hinted row-tile lookup differs at row tile %d (hint %d)", mt, g_prev);
+    }
+    g_prev = a.g;
+    if (mt < capacity) { out[mt * 3] = a.g; out[mt * 3 + 1] = a.row0; out[mt * 3 + 2] = a.rows; }
+  }
+  delete t;
+  return total <= capacity ? 0 : set_error("row tiles need %d entries, capacity %lld", total, (long long)capacity);
+}
+
 int tgg_set_option(const char* key, int value) {
   if (key && strcmp(key, "force_generic") == 0) { g_force_generic = value != 0; return 0; }
   if (key && strcmp(key, "variant") == 0) { set_fast_variant(value); set_fp8_variant(value); return 0; }

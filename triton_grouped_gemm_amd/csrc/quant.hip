@@ -90,8 +90,8 @@ __global__ __launch_bounds__(256) void trans_quant128_kernel(const uint16_t* __r
       if (tid == 0) scales[(int64_t)bn * m_tiles_all + pm] = 0.f;
       continue;
     }
-    const Tile t = sched_tile<128, 128>(p, sm.sched, (int64_t)pm * tiles_n + bn);
-    // sched_tile numbers tiles n-fastest over the real m tiles, so (pm, bn) maps straight through.
+    // The row tile is looked up directly in the group table: the GEMM tile-id order (column chunks) plays no part here.
+    const RowTile t = sched_row_tile<128>(sm.sched, p.G, pm);
     i32x4_t v[8];
     float amax = 0.f;
 #pragma unroll

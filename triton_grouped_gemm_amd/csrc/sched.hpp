@@ -127,9 +127,40 @@ TGG_HD void sched_split(int r, int rows_m, int tiles_n, int nc, int& mt, int& nt
   nt = c * nc + (q - mt * width);
 }
 
+// Row-tile lookup shared by every consumer of the group table (every mode but the K-grouped ones): which group
+// owns the global BM-row tile `mt_glob` (counted over the groups' tiles in order, independent of the tile-id
+// order that sched_tile lays over the (row tile, column tile) space), where its rows start and how many are valid.
 // g_hint: a group at or before the tile's group, if the caller knows one (a workgroup's walk visits tiles in
 // increasing order, and within a column chunk their groups never decrease): the lookup then checks the hinted
 // group and its successor before it falls back to the binary search, each probe being a dependent LDS read.
+struct RowTile {
+  int g;
+  int64_t row0;
+  int rows;
+};
+
+template <int BM, class Table>
+TGG_HD RowTile sched_row_tile(const Table& t, int G, int mt_glob, int g_hint = -1) {
+  int lo = 0, hi = G;  // last g with tile0[g] <= mt_glob
+  if (g_hint >= 0 && g_hint < G && t.tile0[g_hint] <= mt_glob) {
+    lo = g_hint;
+    if (t.tile0[lo + 1] > mt_glob) hi = lo + 1;            // tile0 has G + 1 entries
+    else if (lo + 2 <= G && t.tile0[lo + 2] > mt_glob) { lo = lo + 1; hi = lo + 1; }
+    else lo = lo + 1;                                      // further on: search [lo, G)
+  }
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (t.tile0[mid] <= mt_glob) lo = mid; else hi = mid;
+  }
+  RowTile r;
+  r.g = lo;
+  const int mt = mt_glob - t.tile0[lo];
+  r.row0 = t.row0[lo] + (int64_t)mt * BM;
+  const int left = t.rows[lo] - mt * BM;
+  r.rows = left < BM ? left : BM;
+  return r;
+}
+
 template <int BM, int BN, class Table>
 TGG_HD Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id, int g_hint = -1) {
   Tile r;
@@ -152,23 +183,11 @@ TGG_HD Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id, int
   }
   int mt_glob, nt;
   sched_split(tid32, t.tile0[p.G], tiles_n, nc, mt_glob, nt);
+  const RowTile rt = sched_row_tile<BM>(t, p.G, mt_glob, g_hint);
   r.n0 = nt * BN;
-  int lo = 0, hi = p.G;  // last g with tile0[g] <= mt_glob
-  if (g_hint >= 0 && g_hint < p.G && t.tile0[g_hint] <= mt_glob) {
-    lo = g_hint;
-    if (t.tile0[lo + 1] > mt_glob) hi = lo + 1;            // tile0 has G + 1 entries
-    else if (lo + 2 <= p.G && t.tile0[lo + 2] > mt_glob) { lo = lo + 1; hi = lo + 1; }
-    else lo = lo + 1;                                      // further on: search [lo, G)
-  }
-  while (hi - lo > 1) {
-    const int mid = (lo + hi) >> 1;
-    if (t.tile0[mid] <= mt_glob) lo = mid; else hi = mid;
-  }
-  r.g = lo;
-  const int mt = mt_glob - t.tile0[lo];
-  r.row0 = t.row0[lo] + (int64_t)mt * BM;
-  const int left = t.rows[lo] - mt * BM;
-  r.rows = left < BM ? left : BM;
+  r.g = rt.g;
+  r.row0 = rt.row0;
+  r.rows = rt.rows;
   r.k0 = 0;
   r.k1 = p.K;
   return r;
