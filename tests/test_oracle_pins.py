@@ -156,6 +156,104 @@ def test_cast_recipes_match_torch_expressions():
     assert sz[0, 0] == np.float32(np.float32(1e-4) / np.float32(448.0)) and not cz.any()
 
 
+def test_row_and_expert_cast_recipes_match_torch_expressions():
+    """per_row_cast_to_fp8 / per_expert_cast_to_fp8 against the torch expressions of the reference's
+    per_channel_cast_to_fp8 and per_expert_cast_to_fp8 (gemm/FP8/m_grouped_gemm_channel_expert.py:224-234, :247-261):
+    torch's own fp8 cast and its `fmax / amax` (reciprocal then multiply) stand against the numpy encoder."""
+    for fmt, tdt in (("e4m3fn", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)):
+        fmax = torch.finfo(tdt).max
+        x = _bf16_randn((12, 256), 21, scale=2.5)
+        x[3] = 0.0                       # a whole row at the 1e-4 clamp
+        x[4] *= 1e-3
+        xt = torch.from_numpy(x).to(torch.bfloat16)
+        x = xt.float().numpy()           # the oracle takes fp32 arrays holding bf16 values
+        codes, scales = quant_ref.per_row_cast_to_fp8(x, fmt)
+        v = xt.view(12, -1, 256)
+        amax = v.abs().float().amax(dim=2).view(12, -1).clamp(1e-4)
+        ref = (v * (fmax / amax.unsqueeze(2))).to(tdt).view(12, 256).view(torch.uint8).numpy()
+        assert codes.shape == (12, 256) and scales.shape == (12, 1)
+        assert np.array_equal(codes, ref) and np.array_equal(scales, (amax / fmax).numpy())
+        # the scale is per ROW: scaling one row by 4 changes that row's scale only
+        x2 = x.copy()
+        x2[5] *= 4.0
+        _, s2 = quant_ref.per_row_cast_to_fp8(x2, fmt)
+        assert s2[5, 0] == np.float32(4.0) * scales[5, 0] and np.array_equal(np.delete(s2, 5, 0), np.delete(scales, 5, 0))
+
+        w = _bf16_randn((3, 24, 40), 22, scale=0.3)
+        w[1] *= 8.0
+        wt = torch.from_numpy(w).to(torch.bfloat16)
+        w = wt.float().numpy()
+        cw, sw = quant_ref.per_expert_cast_to_fp8(w, fmt)
+        wv = wt.view(3, 24, 1, 40)
+        wamax = wv.abs().float().amax(dim=(1, 3), keepdim=True).clamp(1e-4)
+        wref = (wv * (fmax / wamax)).to(tdt).view(3, 24, 40).view(torch.uint8).numpy()
+        assert cw.shape == (3, 24, 40) and sw.shape == (3, 1)
+        assert np.array_equal(cw, wref) and np.array_equal(sw, (wamax / fmax).view(3, 1).numpy())
+        assert sw[1, 0] > 4 * sw[0, 0]   # one scale per EXPERT matrix, not a global one
+
+
+def test_fp8_channel_reference_pins():
+    """fp8_channel_reference (gemm/FP8/m_grouped_gemm_channel_expert.py:119-136): unit scales reduce it to gmm;
+    with power-of-two scales folded into integer operands every product is exact, so it must EQUAL the plain
+    per-group matmul of the pre-scaled operands; a brute-force triple loop on a tiny case; scales chosen so that
+    reading b_scale as [N, G] instead of [G, N], or a_scale by group instead of by row, changes the result."""
+    g = torch.Generator().manual_seed(31)
+    sizes = [5, 0, 7]
+    M, K, G, N = 12, 16, 3, 4
+    aq = torch.randint(-6, 7, (M, K), generator=g).float()
+    bq = torch.randint(-6, 7, (G, N, K), generator=g).float()
+    ones_a, ones_b = torch.ones(M, 1), torch.ones(G * N)
+    assert torch.equal(gemm_ref.fp8_channel_reference(aq, ones_a, bq, ones_b, sizes), gemm_ref.gmm(aq, bq, sizes, trans_b=True))
+    sa = 2.0 ** torch.randint(-3, 4, (M, 1), generator=g).float()          # distinct per row
+    sb = 2.0 ** torch.arange(G * N).float().remainder(7).sub(3)            # flattened [G*N], g-major: index g*N + n
+    out = gemm_ref.fp8_channel_reference(aq, sa, bq, sb, sizes)
+    folded = gemm_ref.gmm(aq * sa, bq * sb.view(G, N, 1), sizes, trans_b=True)
+    assert torch.equal(out, folded)
+    wrong = gemm_ref.gmm(aq * sa, bq * sb.view(N, G).t().reshape(G, N, 1), sizes, trans_b=True)
+    assert not torch.equal(out, wrong)                                      # the test can tell [G,N] from [N,G]
+    starts = [0, 5, 5]
+    for gi, (st, sz) in enumerate(zip(starts, sizes)):
+        for r in range(st, st + sz):
+            for n in range(N):
+                acc = sum(float(aq[r, k]) * float(bq[gi, n, k]) for k in range(K))
+                assert float(out[r, n]) == acc * float(sa[r, 0]) * float(sb[gi * N + n])
+    assert gemm_ref.fp8_channel_reference(aq, sa.view(-1), bq, sb, sizes).equal(out)   # [M] and [M,1] scales alike
+
+
+def test_fp8_k_grouped_channel_reference_pins():
+    """fp8_k_grouped_channel_reference (gemm/FP8/k_grouped_gemm_channel_expert.py:104-140: scale element (m, g) at
+    g*M + m, accumulate over the group's token segment, multiply by a_s * b_s^T once at the end)."""
+    g = torch.Generator().manual_seed(32)
+    tokens = [4, 0, 6]
+    M, N, G = 3, 5, 3
+    Kt = sum(tokens)
+    xq = torch.randint(-6, 7, (M, Kt), generator=g).float()
+    yq = torch.randint(-6, 7, (N, Kt), generator=g).float()
+    ones = gemm_ref.fp8_k_grouped_channel_reference(xq, torch.ones(M, G), yq, torch.ones(N, G), tokens)
+    assert ones.shape == (G, M, N)
+    assert torch.equal(ones[0], xq[:, :4] @ yq[:, :4].t()) and torch.count_nonzero(ones[1]) == 0
+    assert torch.equal(ones.sum(0), xq @ yq.t())                            # segments partition the token axis
+    assert torch.equal(ones, gemm_ref.gmm_dw(xq.t().contiguous(), yq.t().contiguous(), tokens))  # == bf16 K-grouped on A^T
+    xs = 2.0 ** torch.randint(-3, 4, (M, G), generator=g).float()
+    ys = 2.0 ** (torch.arange(N * G).float().remainder(5).sub(2)).view(N, G)
+    out = gemm_ref.fp8_k_grouped_channel_reference(xq, xs, yq, ys, tokens)
+    start = 0
+    for gi, t in enumerate(tokens):
+        seg = slice(start, start + t)
+        folded = (xq[:, seg] * xs[:, gi:gi + 1]) @ (yq[:, seg] * ys[:, gi:gi + 1]).t()
+        assert torch.equal(out[gi], folded)
+        for m in range(M):
+            for n in range(N):
+                acc = sum(float(xq[m, k]) * float(yq[n, k]) for k in range(start, start + t))
+                assert float(out[gi, m, n]) == acc * float(xs[m, gi]) * float(ys[n, gi])
+        start += t
+    # the column-major storage the kernel reads (element (m, g) at g*M + m) is what xs[:, g] addresses
+    flat = xs.t().contiguous().view(-1)
+    assert all(float(flat[gi * M + m]) == float(xs[m, gi]) for gi in range(G) for m in range(M))
+    swapped = gemm_ref.fp8_k_grouped_channel_reference(xq, xs.t().reshape(M, G), yq, ys, tokens)
+    assert not torch.equal(swapped, out)
+
+
 # ---- GEMM references: reduce to library routines ----
 def test_gmm_reduces_to_matmul_and_bmm():
     g = torch.Generator().manual_seed(7)
