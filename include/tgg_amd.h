@@ -130,6 +130,16 @@ int tgg_moe_sort_workspace_bytes(int64_t num_tokens, int topk, int num_experts, 
 int tgg_moe_permute_map(const int32_t* indices, int64_t num_tokens, int topk, int num_experts, int64_t num_out_tokens,
                         int32_t* row_id_map, void* tokens_per_expert, int counts_i64, void* workspace,
                         int64_t workspace_bytes, void* stream);
+/* tgg_moe_permute_map without the workspace argument, for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
+ * sort's temporaries live in a fixed 8 MiB + 8 KiB array inside the library's device code (one copy per GPU, held
+ * until the process ends); the call allocates and frees nothing.  Same results as tgg_moe_permute_map.  Limit:
+ * num_tokens * topk <= 1048576 (2^20) assignments, num_experts <= 1024; larger problems are rejected with return
+ * code 1 and a message.  All calls on one GPU share the array: calls that overlap on one GPU (different streams, or
+ * different threads) race; calls on one stream are ordered and safe. */
+int tgg_moe_permute_map_static(const int32_t* indices, int64_t num_tokens, int topk, int num_experts,
+                               int64_t num_out_tokens, int32_t* row_id_map, void* tokens_per_expert, int counts_i64,
+                               void* stream);
 int tgg_moe_permute_rows(const void* input, void* permuted, const int32_t* row_id_map, int64_t num_tokens, int topk,
                          int hidden, int dtype, void* stream);
 int tgg_moe_unpermute(const void* input, void* output, const int32_t* row_id_map, const float* probs,

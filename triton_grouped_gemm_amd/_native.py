@@ -34,6 +34,7 @@ SIGNATURES = {
     "tgg_m_grouped_gemm_fp8_out": [_P, _P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _I, _I, _I, _P],
     "tgg_moe_sort_workspace_bytes": [_L, _I, _I, _P],
     "tgg_moe_permute_map": [_P, _L, _I, _I, _L, _P, _P, _I, _P, _L, _P],
+    "tgg_moe_permute_map_static": [_P, _L, _I, _I, _L, _P, _P, _I, _P],
     "tgg_moe_permute_rows": [_P, _P, _P, _L, _I, _I, _I, _P],
     "tgg_moe_unpermute": [_P, _P, _P, _P, _L, _I, _I, _I, _P],
     "tgg_moe_unpermute_bwd": [_P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _P],

@@ -342,6 +342,18 @@ int tgg_moe_permute_map(const int32_t* indices, int64_t num_tokens, int topk, in
                                 counts_i64, workspace, (hipStream_t)stream);
 }
 
+int tgg_moe_permute_map_static(const int32_t* indices, int64_t num_tokens, int topk, int num_experts,
+                               int64_t num_out_tokens, int32_t* row_id_map, void* tokens_per_expert, int counts_i64,
+                               void* stream) {
+  if (num_tokens < 0 || topk < 1) return set_error("bad num_tokens / topk");
+  if (num_tokens >= (1ll << 31) / topk) return set_error("num_tokens * topk must stay below 2^31");
+  if (num_experts < 1 || num_experts > 1024) return set_error("num_experts=%d outside [1, 1024]", num_experts);
+  if (num_tokens > 0 && (!indices || !row_id_map)) return set_error("null pointer");
+  const int64_t capacity = num_out_tokens > 0 ? num_out_tokens : num_tokens * topk;
+  return launch_moe_permute_map_static(indices, num_tokens, topk, num_experts, capacity, row_id_map, tokens_per_expert,
+                                       counts_i64, (hipStream_t)stream);
+}
+
 int tgg_moe_permute_rows(const void* input, void* permuted, const int32_t* row_id_map, int64_t num_tokens, int topk,
                          int hidden, int dtype, void* stream) {
   int64_t rb;

@@ -24,6 +24,9 @@ int launch_fast_fp8_block(const GemmParams& p, hipStream_t s);
 int64_t moe_sort_workspace_bytes(int64_t n, int num_experts);
 int launch_moe_permute_map(const int32_t* indices, int64_t tokens, int topk, int num_experts, int64_t capacity,
                            int32_t* row_id_map, void* counts, int counts_i64, void* workspace, hipStream_t s);
+int64_t moe_static_max_assignments();
+int launch_moe_permute_map_static(const int32_t* indices, int64_t tokens, int topk, int num_experts, int64_t capacity,
+                                  int32_t* row_id_map, void* counts, int counts_i64, hipStream_t s);
 int launch_moe_permute_rows(const void* in, void* out, const int32_t* row_id_map, int64_t tokens, int topk,
                             int64_t row_bytes, hipStream_t s);
 int launch_moe_unpermute(const void* in, void* out, const int32_t* row_id_map, const float* prob, int64_t tokens,

@@ -15,6 +15,8 @@
 //   permute_rows    reads each token row once and writes it to its up to topK destinations
 //   unpermute       out[t] = sum_k prob[t,k] * in[row_id_map[k,t]]
 //   unpermute_bwd   act_grad[dest] = prob[t,k] * grad[t];  prob_grad[t,k] = <grad[t], fwd_in[dest]>
+#include <mutex>
+
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -325,6 +327,56 @@ int launch_moe_permute_map(const int32_t* indices, int64_t tokens, int topk, int
   hipLaunchKernelGGL(moe_place_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, indices, n, tokens, topk,
                      num_experts, chunks, capacity, w.table, w.expert_start, w.rank, row_id_map);
   return check_launch("moe_permute_map");
+}
+
+// ---- the sort without a caller-provided workspace ---------------------------------------------------------------
+// For callers that cannot allocate (HIP graph capture, serving loops): the sort's temporaries live in a fixed
+// array in device memory that is part of the library's code object.  Sized for the largest problem the entry point
+// accepts: 2^20 assignments, 1024 experts (table 4 MiB + rank 4 MiB + two 4 KiB expert rows).  Every GPU the
+// library runs on holds its own copy at its own address until the process ends; all calls on one GPU share it, so
+// calls that overlap on one GPU (different streams) race.  Nothing in it has to start at zero: the counting pass
+// writes every table entry and rank it later reads, the scans write totals and starts.
+constexpr int64_t kStaticMaxAssignments = 1ll << 20;
+constexpr size_t kStaticScratchBytes = (size_t)kMaxExperts * (kStaticMaxAssignments / kChunk) * 4 + 2 * (size_t)kMaxExperts * 4 +
+                                       (size_t)kStaticMaxAssignments * 4;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of this GPU's copy of `scratch`, looked up once per device (the array's name is only a host-side
+// handle for hipGetSymbolAddress; it is never passed to a kernel or a memory call).
+static int static_scratch_ptr(void** out) {
+  static std::mutex mu;
+  static void* ptr[64] = {nullptr};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return check_launch("hipGetDevice");
+  if (dev < 0 || dev >= 64) return set_error("device ordinal %d outside [0, 64)", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptr[dev]) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return set_error("hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+    }
+    ptr[dev] = p;
+  }
+  *out = ptr[dev];
+  return 0;
+}
+
+int64_t moe_static_max_assignments() { return kStaticMaxAssignments; }
+
+int launch_moe_permute_map_static(const int32_t* indices, int64_t tokens, int topk, int num_experts, int64_t capacity,
+                                  int32_t* row_id_map, void* counts, int counts_i64, hipStream_t s) {
+  const int64_t n = tokens * topk;
+  if (n > kStaticMaxAssignments)
+    return set_error("num_tokens * topk = %lld exceeds the %lld assignments the built-in scratch array holds; "
+                     "use tgg_moe_permute_map with a workspace", (long long)n, (long long)kStaticMaxAssignments);
+  if (carve(nullptr, n, num_experts).bytes > kStaticScratchBytes)
+    return set_error("sort temporaries of %zu bytes exceed the built-in scratch array (%zu bytes)",
+                     carve(nullptr, n, num_experts).bytes, kStaticScratchBytes);
+  void* ws = nullptr;
+  if (int e = static_scratch_ptr(&ws)) return e;
+  return launch_moe_permute_map(indices, tokens, topk, num_experts, capacity, row_id_map, counts, counts_i64, ws, s);
 }
 
 int launch_moe_permute_rows(const void* in, void* out, const int32_t* row_id_map, int64_t tokens, int topk,
