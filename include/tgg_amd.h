@@ -60,7 +60,8 @@ int tgg_m_grouped_gemm_fp8_channel(const void* Aq, const float* a_scale, const v
                                    int fmt_a, int fmt_b, int out_dtype, int num_cu, void* stream);
 
 /* out[g] = (x[:,seg_g] . y[:,seg_g]^T) * xs[g*M+m] * ys[g*N+n], x [M,Ktot], y [N,Ktot], segments =
- * prefix sums of tokens[g]; bf16 output [G,M,N].  Replaces matmul
+ * prefix sums of tokens[g]; bf16 output [G,M,N].  Any token counts (the reference wants them padded to 128 with
+ * zero data; here a segment ends where its count says); Ktot must be a multiple of 16.  Replaces matmul
  * (gemm/FP8/k_grouped_gemm_channel_expert.py:143-181). */
 int tgg_k_grouped_gemm_fp8_channel(const void* x, const float* xs, const void* y, const float* ys, void* out,
                                    const int32_t* tokens, int G, int M, int N, int64_t Ktot, int fmt_a, int fmt_b,
@@ -174,7 +175,10 @@ int tgg_debug_row_tiles(const int64_t* sizes, int G, int mode, int64_t m_total, 
  *                        workgroups, 256x256 otherwise; 1 = always 256x128; 2 = always 256x256
  *   "tile_split"    0/1  M-grouped tuned kernels: per-XCD contiguous tile ranges (default 1) or interleaved sweeps
  *   "n_chunk"       int  column tiles per chunk of the tile order (0 = automatic, at most eight)
- *   "store_nt"      0/1  write the output with non-temporal stores (default 1) */
+ *   "store_nt"      0/1  write the output with non-temporal stores (default 1)
+ *   "kg_second_launch" 0/1  tgg_k_grouped_gemm_fp8_channel enqueues the tuned kernel and the shape-agnostic kernel, and
+ *                        each decides on the device from the token counts whether it runs (tuned: all counts multiples
+ *                        of 16); 0 leaves the second one out, so a test can see what the tuned kernel does alone */
 int tgg_set_option(const char* key, int value);
 const char* tgg_last_error(void);
 int tgg_version(void);

@@ -115,6 +115,70 @@ def test_fp8_k_grouped_channel(dev, variant, dtype_a, dtype_b):
     assert rd <= FP8_RDIFF and rd <= 2.0 ** -7, rd
 
 
+def _k_grouped_unpadded_case(tokens, M, N, seed):
+    """Per-expert blocks quantised per row (one scale per row and expert) and laid side by side WITHOUT padding."""
+    xq_l, xs_l, yq_l, ys_l = [], [], [], []
+    for i, t in enumerate(tokens):
+        if t == 0:
+            xq, xs = np.zeros((M, 0), np.uint8), np.full((M, 1), 1e-4 / 448, np.float32)
+            yq, ys = np.zeros((N, 0), np.uint8), np.full((N, 1), 1e-4 / 448, np.float32)
+        else:
+            xq, xs = quant_ref.per_row_cast_to_fp8(to_np_f32(_randn((M, t), seed + i)))
+            yq, ys = quant_ref.per_row_cast_to_fp8(to_np_f32(_randn((N, t), seed + 50 + i)))
+        xq_l.append(xq); xs_l.append(xs); yq_l.append(yq); ys_l.append(ys)
+    return np.concatenate(xq_l, 1), np.concatenate(xs_l, 1), np.concatenate(yq_l, 1), np.concatenate(ys_l, 1)
+
+
+@pytest.mark.parametrize("tokens,tuned_runs", [
+    ([125, 300, 0, 128, 7], False),      # not multiples of 16: the shape-agnostic kernel takes the call
+    ([112, 304, 0, 128, 16], True),      # multiples of 16, not of 128: the tuned kernel cuts every group's last slab
+    ([128, 384, 0, 256], True),
+    ([16, 16, 16, 0, 48], True),
+])
+@pytest.mark.parametrize("M,N", [(136, 264), (512, 256)])
+def test_fp8_channel_k_grouped_unpadded_counts(dev, tokens, tuned_runs, M, N):
+    """Token counts as they are (the reference pads every expert to 128 with zero data,
+    gemm/FP8/k_grouped_gemm_channel_expert.py:238-260; here a segment simply ends where its count says): tuned and
+    shape-agnostic path against the oracle, and the device-side choice between them seen from outside."""
+    G, Kt = len(tokens), sum(tokens)
+    xq, xs, yq, ys = _k_grouped_unpadded_case(tokens, M, N, 60)
+    ref = gemm_ref.fp8_k_grouped_channel_reference(torch.from_numpy(quant_ref.dequant(xq)), torch.from_numpy(xs),
+                                                   torch.from_numpy(quant_ref.dequant(yq)), torch.from_numpy(ys), tokens)
+    args = (_codes_to_torch(xq, "e4m3fn").to(dev), torch.from_numpy(xs).to(dev), _codes_to_torch(yq, "e4m3fn").to(dev),
+            torch.from_numpy(ys).to(dev), torch.tensor(tokens, dtype=torch.int32, device=dev), M, N, Kt, G)
+    outs = {}
+    for name, opts in (("default", {}), ("generic", {"force_generic": 1}), ("tuned_only", {"kg_second_launch": 0})):
+        for k, v in opts.items():
+            _native.set_option(k, v)
+        try:
+            if name == "tuned_only":
+                # call the C ABI on a sentinel-filled output to see whether the tuned kernel ran
+                out = torch.full((G, M, N), -77.0, dtype=torch.bfloat16, device=dev)
+                xs_e = args[1].t().contiguous()
+                ys_e = args[3].t().contiguous()
+                _native.call("tgg_k_grouped_gemm_fp8_channel", args[0].data_ptr(), xs_e.data_ptr(), args[2].data_ptr(),
+                             ys_e.data_ptr(), out.data_ptr(), args[4].data_ptr(), G, M, N, Kt, _native.E4M3, _native.E4M3,
+                             -1, _native.stream_of(out))
+                torch.cuda.synchronize()
+            else:
+                out = matmul(*args)
+        finally:
+            for k in opts:
+                _native.set_option(k, 1 if k == "kg_second_launch" else 0)
+        outs[name] = out.cpu().float()
+    for name in ("default", "generic"):
+        rd = gemm_ref.rdiff(outs[name], ref)
+        assert rd <= FP8_RDIFF and rd <= 2.0 ** -7, (name, rd)
+        for g, t in enumerate(tokens):
+            if t == 0:
+                assert torch.count_nonzero(outs[name][g]) == 0
+    if tuned_runs:
+        assert torch.equal(outs["tuned_only"], outs["default"])
+    else:
+        assert bool((outs["tuned_only"] == -77.0).all())      # the tuned kernel saw the counts and left
+        assert torch.equal(outs["default"], outs["generic"])  # ... to the shape-agnostic kernel
+
+
 def _block_scaled_case(sizes, N, K, seed):
     padded = [(s + 127) // 128 * 128 for s in sizes]
     Mp, G = sum(padded), len(sizes)

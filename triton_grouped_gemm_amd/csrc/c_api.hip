@@ -15,6 +15,7 @@ static int g_force_generic = 0;
 static int g_tile_split = 1;
 static int g_store_nt = 1;
 static int g_n_chunk = 0;
+static int g_kg_second_launch = 1;
 
 int set_error(const char* fmt, ...) {
   va_list ap;
@@ -244,7 +245,14 @@ int tgg_k_grouped_gemm_fp8_channel(const void* x, const float* xs, const void* y
   p.mode = MODE_KG_COUNT; p.m_total = M; p.k_total = Ktot; p.N = N; p.K = 0;
   p.a_sm = Ktot; p.a_sk = 1; p.b_sg = 0; p.b_sn = Ktot; p.b_sk = 1; p.c_sg = (int64_t)M * N;
   p.grid_limit = num_cu;
-  if (!g_force_generic && fast_fp8_supported(p, false)) return launch_fast_fp8_channel(p, fmt_a, fmt_b, TGG_BF16, (hipStream_t)stream);
+  if (!g_force_generic && fast_fp8_supported(p, false)) {
+    // The tuned kernel needs every token count to be a multiple of 16 and only the device knows the counts: both
+    // kernels are enqueued, each reads the counts first and exactly one of them runs (the other returns at once).
+    p.kg_gate = 1;
+    if (int e = launch_fast_fp8_channel(p, fmt_a, fmt_b, TGG_BF16, (hipStream_t)stream)) return e;
+    if (!g_kg_second_launch) return 0;
+    p.kg_gate = 2;
+  }
   return launch_generic_fp8_channel(p, fmt_a, fmt_b, TGG_BF16, (hipStream_t)stream);
 }
 
@@ -457,6 +465,7 @@ int tgg_set_option(const char* key, int value) {
   if (key && strcmp(key, "variant") == 0) { set_fast_variant(value); set_fp8_variant(value); return 0; }
   if (key && strcmp(key, "tile_split") == 0) { g_tile_split = value != 0; return 0; }
   if (key && strcmp(key, "n_chunk") == 0) { g_n_chunk = value < 0 ? 0 : value; return 0; }
+  if (key && strcmp(key, "kg_second_launch") == 0) { g_kg_second_launch = value != 0; return 0; }
   if (key && strcmp(key, "store_nt") == 0) { g_store_nt = value != 0; return 0; }
   return set_error("unknown option '%s'", key ? key : "(null)");
 }

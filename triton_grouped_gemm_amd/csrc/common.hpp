@@ -97,6 +97,11 @@ struct GemmParams {
   int tile_split;         // tuned kernels: 1 = per-XCD contiguous tile ranges (see sched_walk)
   int n_chunk;            // column tiles per chunk of the tile order, 0 = automatic (see sched_tile)
   int store_nt;           // tuned kernels: 1 = non-temporal output stores
+  // FP8 K-grouped by token counts: the tuned kernel copies 16-byte chunks, so it needs every count (hence every
+  // segment start) to be a multiple of 16; the shape-agnostic kernel takes anything.  Only the device knows the
+  // counts, so both kernels are launched and each looks at the counts first: 1 = run only if all counts are
+  // multiples of 16 (tuned), 2 = run only if one is not (shape-agnostic), 0 = always run.
+  int kg_gate;
   // fused 1x128 quantisation of the output (tuned 16-bit M-grouped kernels): C then holds fp8 codes [rows, N] and
   // the scale of (row, 128-column block) goes to q_scales[row * q_rs + block * q_bs]
   float* q_scales;

@@ -80,6 +80,10 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   const int tail_chunks = KGROUP ? 0 : (p.K % BKB) / 16;
   const int a_voff_tail = OpA::lane_chunk(lane, wave % OpA::NPAT) >= tail_chunks ? kNoFetch : a_voff;
   const int b_voff_tail = OpB::lane_chunk(lane, wave % OpB::NPAT) >= tail_chunks ? kNoFetch : b_voff;
+  // K-grouped: a group's last slab holds only the group's remaining tokens (a multiple of 16, see kg_gate); the
+  // chunks beyond them belong to the next group and are not fetched
+  const int a_chunk = OpA::lane_chunk(lane, wave % OpA::NPAT);
+  const int b_chunk = OpB::lane_chunk(lane, wave % OpB::NPAT);
   const int kblocks = (p.K + 127) >> 7;
   const int nblocks = (p.N + 127) >> 7;
 
@@ -105,6 +109,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
     uint64_t a_base, b_base, s_base;
     int a_left, b_left;  // operand windows stay below 2^30 bytes: 32-bit scalar bookkeeping
     int s_bytes, kt_n, issued;
+    int k_left;  // K-grouped: bytes of the group's token range not yet issued
   };
   auto slabs_of = [&](const Tile& t) -> int { return KGROUP ? (int)((t.k1 - t.k0 + BKB - 1) / BKB) : (p.K + BKB - 1) / BKB; };
   auto make_io = [&](const Tile& t) {
@@ -121,6 +126,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
     io.s_base = BLOCK ? uniform64((uint64_t)(p.sa + t.row0)) : 0;
     io.s_bytes = BLOCK ? __builtin_amdgcn_readfirstlane(a_rows * 4) : 0;
     io.issued = 0;
+    io.k_left = KGROUP ? __builtin_amdgcn_readfirstlane((int)(t.k1 - t.k0)) : 0;
     return io;
   };
   // Weight scales of this wave's column block for every slab of a tile: lane kb holds block kb.
@@ -149,6 +155,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
     feed.a_base = feed.b_base = feed.s_base = (uint64_t)p.A;
     feed.a_left = feed.b_left = 0;
     feed.s_bytes = 0;
+    feed.k_left = 0;
     for (; id < walk.end; id += walk.stride) {
       const Tile tt = id == nt_id ? nt : sched_tile<C::BM, C::BN>(p, sched, id);
       if (slabs_of(tt) > 0) {
@@ -162,6 +169,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
     i32x4_t ra, rb, rs;
     uint32_t base;
     bool tail;  // the tile's last slab, cut short by K
+    int chunks; // K-grouped: 16-byte chunks of this slab that belong to the group (8 but for a group's last slab)
   };
   constexpr int CA = C::NI_A / C::NWAVES, CB = C::NI_B / C::NWAVES, CS = BLOCK ? 1 : 0, NC = CS + CA + CB;
   auto begin_slab = [&](int buf) {
@@ -172,6 +180,8 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
     sc.rs = make_rsrc32(feed.s_base, live ? feed.s_bytes : 0);
     sc.base = smem_addr + buf * C::STAGE_BYTES;
     sc.tail = tail_chunks != 0 && feed.issued + 1 == feed.kt_n;
+    sc.chunks = KGROUP ? (feed.k_left >= BKB ? 8 : (feed.k_left > 0 ? feed.k_left >> 4 : 0)) : 8;
+    feed.k_left -= BKB;
     feed.a_base += BKB;
     feed.a_left -= BKB;
     feed.b_base += BKB;
@@ -190,10 +200,12 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
                       mine ? (wave * 64 + lane) * 4 : kNoFetch);
     } else if (k < CS + CA) {
       const int idx = wave + (k - CS) * C::NWAVES;  // wave-uniform
-      copy_b128_to_lds(sc.ra, sc.base + idx * 1024, (sc.tail ? a_voff_tail : a_voff) + idx * OpA::RPI * (int)ld);
+      const int v0 = KGROUP ? (a_chunk >= sc.chunks ? kNoFetch : a_voff) : (sc.tail ? a_voff_tail : a_voff);
+      copy_b128_to_lds(sc.ra, sc.base + idx * 1024, v0 + idx * OpA::RPI * (int)ld);
     } else {
       const int idx = wave + (k - CS - CA) * C::NWAVES;
-      copy_b128_to_lds(sc.rb, sc.base + C::A_BYTES + idx * 1024, (sc.tail ? b_voff_tail : b_voff) + idx * OpB::RPI * (int)ld);
+      const int v0 = KGROUP ? (b_chunk >= sc.chunks ? kNoFetch : b_voff) : (sc.tail ? b_voff_tail : b_voff);
+      copy_b128_to_lds(sc.rb, sc.base + C::A_BYTES + idx * 1024, v0 + idx * OpB::RPI * (int)ld);
     }
   };
 
@@ -446,7 +458,9 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
 template <class C, int FA, int FB, int EPI, int OUT, bool KGROUP>
 __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  sched_init<C::BM>(p, *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::SCHED_OFF));
+  auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::SCHED_OFF);
+  sched_init<C::BM>(p, sched);
+  if (KGROUP && !sched_kg_gate_open(p, sched)) return;
   gemm_fp8_body<C, FA, FB, EPI, OUT, KGROUP, C::SCHED_OFF, false>(p);
 }
 
@@ -533,14 +547,14 @@ int launch_channel_fmt(const GemmParams& p, int ta, int tb, int out_dt, hipStrea
 
 void set_fp8_variant(int v) { g_fp8_variant = v; }
 
-// K-contiguous fp8 operands with every reduction range a multiple of the 128-deep slab.
+// K-contiguous fp8 operands; K-grouped: token counts that are multiples of 16 (checked on the device, see kg_gate).
 bool fast_fp8_supported(const GemmParams& p, bool block_scaled) {
   if (p.G > kFastMaxGroups) return false;
   if ((p.N & 7) != 0) return false;
   const bool kgroup = p.mode == MODE_KG_COUNT;
   if (kgroup) {
     if (block_scaled) return false;
-    return (p.k_total % BKB) == 0 && p.k_total * 256 < (1ll << 30);
+    return (p.k_total % 16) == 0 && p.k_total * 256 < (1ll << 30);
   }
   if (p.mode != MODE_MG && p.mode != MODE_MG_PAD) return false;
   if (p.K < 16 || (p.K & 15) != 0) return false;

@@ -140,6 +140,7 @@ __global__ __launch_bounds__(GTHREADS) void gemm_generic_kernel(const GemmParams
   __shared__ GenericSmem sm;
   constexpr int ESA = ElemSize<TA>::v, ESB = ElemSize<TB>::v;
   sched_init<GBM>(p, sm.sched);
+  if (!sched_kg_gate_open(p, sm.sched)) return;
   const int64_t num_tiles = sched_num_tiles<GBM, GBN>(p, sm.sched);
   const bool kmode = (p.mode == MODE_KG || p.mode == MODE_KG_COUNT);
 

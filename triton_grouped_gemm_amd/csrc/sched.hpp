@@ -89,6 +89,17 @@ TGG_DEV void sched_init(const GemmParams& p, Table& t) {
   __syncthreads();
 }
 
+// K-grouped by counts: does the launch pass its gate (GemmParams::kg_gate)?  All threads of the workgroup must call
+// this after sched_init; the answer is the same in every workgroup of the launch.
+template <class Table>
+TGG_DEV bool sched_kg_gate_open(const GemmParams& p, const Table& t) {
+  if (p.kg_gate == 0) return true;
+  int bad = 0;
+  for (int g = threadIdx.x; g < p.G; g += blockDim.x) bad |= (t.rows[g] & 15) != 0;
+  const int n_bad = __syncthreads_count(bad);
+  return p.kg_gate == 1 ? n_bad == 0 : n_bad != 0;
+}
+
 template <int BM, int BN, class Table>
 TGG_HD int64_t sched_num_tiles(const GemmParams& p, const Table& t) {
   const int tiles_n = (p.N + BN - 1) / BN;
