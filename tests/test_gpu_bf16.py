@@ -23,11 +23,15 @@ def _ints(shape, seed, dtype=torch.bfloat16, lo=-1, hi=1):
     return torch.randint(lo, hi + 1, shape, generator=g).to(dtype)
 
 
-@pytest.fixture(params=[0, 1], ids=["tuned", "generic"])
+@pytest.fixture(params=[0, 1, 2], ids=["tuned", "generic", "four_wave"])
 def variant(request, dev):
-    _native.set_option("force_generic", request.param)
+    """tuned: what a call gets by default; generic: the shape-agnostic kernel; four_wave: the large-problem kernel
+    forced onto every M-grouped NT shape it can take, whatever the size (other calls run as in `tuned`)."""
+    _native.set_option("force_generic", int(request.param == 1))
+    _native.set_option("four_wave", 2 if request.param == 2 else 0)
     yield request.param
     _native.set_option("force_generic", 0)
+    _native.set_option("four_wave", 0)
 
 
 def test_config1_tiny_reference_case(dev, variant):

@@ -53,6 +53,13 @@ def test_tuned_equals_generic_on_random_shapes(dev, seed):
             a = (torch.randn(M, K, device=dev) * K ** -0.5).to(dt)
             b = torch.randn((G, N, K) if tb else (G, K, N), device=dev).to(dt)
             out, ref = _both(lambda: m_grouped_gemm(a, b, st, tb))
+            if tb:  # the four-wave kernel, forced onto this size, must give the same bits
+                _native.set_option("four_wave", 2)
+                try:
+                    out4 = m_grouped_gemm(a, b, st, tb)
+                finally:
+                    _native.set_option("four_wave", 0)
+                assert torch.equal(out4, ref), f"four-wave kernel differs: seed {seed} case {case} G={G} N={N} K={K} {dt}"
         elif kind == 1 and M > 0:
             Md = 8 * rng.randint(1, 80)
             a = torch.randn(M, Md, device=dev).to(dt)

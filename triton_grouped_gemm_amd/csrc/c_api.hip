@@ -16,6 +16,7 @@ static int g_tile_split = 1;
 static int g_store_nt = 1;
 static int g_n_chunk = 0;
 static int g_kg_second_launch = 1;
+static int g_four_wave = 0;  // 0 = eight-wave kernels only, 1 = four-wave kernel on large M-grouped NT launches, 2 = on every launch it can take
 
 int set_error(const char* fmt, ...) {
   va_list ap;
@@ -50,6 +51,8 @@ int launch_block_cast128(const void*, void*, float*, int, int, int, int, hipStre
 int launch_cvt_fp8(const float*, void*, int64_t, int, hipStream_t);
 bool fast_supported(const GemmParams& p, int dt, int layout);
 int launch_fast_16bit(const GemmParams& p, int dt, int layout, hipStream_t s);
+bool w4_supported(const GemmParams& p, int dt, int layout, bool any_size);
+int launch_w4_16bit(const GemmParams& p, int dt, int layout, hipStream_t s);
 bool fast_quant_supported(const GemmParams& p, int dt, int layout);
 int launch_fast_16bit_quant(const GemmParams& p, int dt, int layout, hipStream_t s);
 void set_fast_variant(int v);
@@ -76,6 +79,7 @@ static GemmParams zero_params() {
 }
 
 static int dispatch_16bit(const GemmParams& p, int dt, int layout, hipStream_t s) {
+  if (!g_force_generic && g_four_wave && w4_supported(p, dt, layout, g_four_wave == 2)) return launch_w4_16bit(p, dt, layout, s);
   if (!g_force_generic && fast_supported(p, dt, layout)) return launch_fast_16bit(p, dt, layout, s);
   return launch_generic_16bit(p, dt, layout, s);
 }
@@ -466,6 +470,7 @@ int tgg_set_option(const char* key, int value) {
   if (key && strcmp(key, "tile_split") == 0) { g_tile_split = value != 0; return 0; }
   if (key && strcmp(key, "n_chunk") == 0) { g_n_chunk = value < 0 ? 0 : value; return 0; }
   if (key && strcmp(key, "kg_second_launch") == 0) { g_kg_second_launch = value != 0; return 0; }
+  if (key && strcmp(key, "four_wave") == 0) { g_four_wave = value < 0 ? 0 : (value > 2 ? 2 : value); return 0; }
   if (key && strcmp(key, "store_nt") == 0) { g_store_nt = value != 0; return 0; }
   return set_error("unknown option '%s'", key ? key : "(null)");
 }
