@@ -6,7 +6,10 @@ operands are already resident in HBM.  Prints ONE JSON line: TFLOP/s = 2*M*N*K /
 roofline fraction of the GEMM kernel (HIP-event timed on the launch stream) and, beside it, the
 reference's per-group torch matmul timed on this box's host cores over a bounded sample of groups.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+With no flags the same run also times the FP8 block-scaled M-grouped configuration (the other half of the
+headline metric) and reports it under the "fp8" key of the line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--uniform-groups] [--no-cpu-baseline]
 """
 from __future__ import annotations
 
@@ -64,15 +67,40 @@ WORKLOADS = {
 }
 
 
-def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu: int = -1):
+METRICS = {
+    "mg": "grouped GEMM TFLOP/s (2*M*N*K/time), BF16 M-grouped G=128",
+    "mgq": "grouped GEMM TFLOP/s (2*M*N*K/time), BF16 M-grouped G=128, output quantised 1x128 in the epilogue",
+    "masked": "grouped GEMM TFLOP/s (2*valid_rows*N*K/time), BF16 masked M-grouped G=128",
+    "kg": "grouped GEMM TFLOP/s (2*K_total*M*N/time), BF16 K-grouped G=128",
+    "fp8": "grouped GEMM TFLOP/s (2*M*N*K/time), FP8 block-scaled M-grouped G=128",
+    "fp8c": "grouped GEMM TFLOP/s (2*M*N*K/time), FP8 per-channel M-grouped G=128",
+    "fp8ck": "grouped GEMM TFLOP/s (2*K_total*M*N/time), FP8 per-channel K-grouped G=128",
+    "quant": "transposing 128x128 quantizer, algorithmic GB/s",
+    "permute": "MoE permute (sort + row mover), algorithmic GB/s",
+    "unpermute": "MoE unpermute, algorithmic GB/s",
+}
+
+
+def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu: int = -1, uniform: bool = False,
+                   groups: int = None, m_total: int = None):
     """Returns (fn, flops_per_step, algorithmic_bytes_per_step, dtype_tag, description, cpu_sample_fn); leaves a
-    per-group library-GEMM loop over the same operands in ``build_workload.vendor_loop`` where one exists."""
+    per-group library-GEMM loop over the same operands in ``build_workload.vendor_loop`` where one exists, the
+    tensor that loop writes in ``build_workload.vendor_out`` and the operands in ``build_workload.operands``.
+    ``uniform``: every group gets m_total / groups rows (the reference's published tables use 128 groups of 5120
+    rows) instead of the Dirichlet-multinomial draw.  ``groups`` / ``m_total`` shrink the problem (tests)."""
     build_workload.vendor_loop = None
+    build_workload.vendor_out = None
+    build_workload.vendor_kind = None
+    build_workload.operands = {}
     from triton_grouped_gemm_amd import workloads as wl
     from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm_TMA import m_grouped_gemm
     kind, N, K, trans_b = WORKLOADS[name]
-    sizes_cpu = wl.dirichlet_multinomial_sizes(G, M_TOTAL, 128, seed=seed)
+    G = groups or globals()["G"]
+    M_TOTAL = m_total or globals()["M_TOTAL"]
+    sizes_cpu = wl.uniform_sizes(G, M_TOTAL) if uniform else wl.dirichlet_multinomial_sizes(G, M_TOTAL, 128, seed=seed)
     sizes = sizes_cpu.to(dev)
+    size_tag = f"uniform, {M_TOTAL // G} rows per group" if uniform else "dirichlet-multinomial, 128-aligned"
+    bounds = [(int(s0), int(s0 + n)) for s0, n in zip((sizes_cpu.cumsum(0) - sizes_cpu).tolist(), sizes_cpu.tolist())]
     if kind == "mg":
         a = wl.randn_bf16((M_TOTAL, K), K ** -0.5, seed + 1, dev)
         b = wl.randn_bf16((G, N, K) if trans_b else (G, K, N), K ** -0.5, seed + 2, dev)
@@ -106,7 +134,6 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
                 if t_used >= budget_s:
                     break
             return done_flops / t_used / 1e12, f"{groups} largest groups of {G} ({done_flops / flops * 100:.1f}% of the step's flops), bf16 torch matmul per group"
-        bounds = [(int(s0), int(s0 + n)) for s0, n in zip((sizes_cpu.cumsum(0) - sizes_cpu).tolist(), sizes_cpu.tolist())]
         c_ref = torch.empty((M_TOTAL, N), device=dev, dtype=torch.bfloat16)
 
         def vendor_loop():  # one library GEMM per expert, the GPU baseline the reference's tables compare against
@@ -114,8 +141,9 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
                 if s1 > s0:
                     torch.matmul(a[s0:s1], b[g].t() if trans_b else b[g], out=c_ref[s0:s1])
         build_workload.vendor_loop = vendor_loop
+        build_workload.vendor_out = c_ref
         return fn, flops, nbytes, "bf16", dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, trans_b=trans_b,
-                                               group_sizes="dirichlet-multinomial, 128-aligned", seed=seed), cpu_sample
+                                               group_sizes=size_tag, seed=seed), cpu_sample
     if kind == "mgq":
         from triton_grouped_gemm_amd.gemm.fused import m_grouped_gemm_fp8_out
         a = wl.randn_bf16((M_TOTAL, K), K ** -0.5, seed + 1, dev)
@@ -124,7 +152,7 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
         nbytes = 2.0 * M_TOTAL * K + 2.0 * G * N * K + 1.0 * M_TOTAL * N + 4.0 * M_TOTAL * N / 128
         return (fn, 2.0 * M_TOTAL * N * K, nbytes, "bf16",
                 dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, trans_b=trans_b, output="e4m3fn codes + 1x128 fp32 scales",
-                     group_sizes="dirichlet-multinomial, 128-aligned", seed=seed), None)
+                     group_sizes=size_tag, seed=seed), None)
     if kind == "masked":
         from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm_masked_TMA import m_grouped_gemm_masked
         m_max = 512
@@ -143,7 +171,6 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
         a = wl.randn_bf16((M_TOTAL, Md), 1.0, seed + 1, dev)
         b = wl.randn_bf16((M_TOTAL, Nd), 1.0, seed + 2, dev)
         fn = lambda: k_grouped_gemm(a, b, sizes)
-        bounds = [(int(s0), int(s0 + n)) for s0, n in zip((sizes_cpu.cumsum(0) - sizes_cpu).tolist(), sizes_cpu.tolist())]
         c_ref = torch.zeros((G, Md, Nd), device=dev, dtype=torch.bfloat16)
 
         def vendor_loop():
@@ -151,8 +178,9 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
                 if s1 > s0:
                     torch.matmul(a[s0:s1].t(), b[s0:s1], out=c_ref[g])
         build_workload.vendor_loop = vendor_loop
+        build_workload.vendor_out = c_ref
         return (fn, 2.0 * M_TOTAL * Md * Nd, 2.0 * M_TOTAL * (Md + Nd) + 2.0 * G * Md * Nd, "bf16",
-                dict(workload=name, G=G, K_total=M_TOTAL, M_dim=Md, N_dim=Nd, seed=seed), None)
+                dict(workload=name, G=G, K_total=M_TOTAL, M_dim=Md, N_dim=Nd, group_sizes=size_tag, seed=seed), None)
     if kind == "fp8":
         from triton_grouped_gemm_amd.gemm.deep_gemm_ops import m_grouped_fp8_nt_contiguous
         from triton_grouped_gemm_amd.quant.fp8_cast import per_block_cast_to_fp8, per_token_cast_to_fp8
@@ -165,8 +193,20 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
         out = torch.empty((M_TOTAL, N), device=dev, dtype=torch.bfloat16)
         fn = lambda: m_grouped_fp8_nt_contiguous(aq, wq, sizes, out=out)
         nbytes = M_TOTAL * K + 4.0 * M_TOTAL * K / 128 + G * N * K + 4.0 * G * (N / 128) * (K / 128) + 2.0 * M_TOTAL * N
+        build_workload.operands = dict(aq=aq, wq=wq, out=out, sizes=sizes)
+        c_ref = torch.empty((M_TOTAL, N), device=dev, dtype=torch.bfloat16)
+        one = torch.ones((), device=dev, dtype=torch.float32)
+
+        def vendor_loop():  # one library FP8 GEMM per expert on the same codes; it applies NO block scales
+            for g, (s0, s1) in enumerate(bounds):
+                if s1 > s0:
+                    c_ref[s0:s1] = torch._scaled_mm(aq[0][s0:s1], wq[0][g].t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16)
+        build_workload.vendor_loop = vendor_loop
+        build_workload.vendor_out = c_ref
+        build_workload.vendor_kind = "torch._scaled_mm per group (hipBLASLt), same fp8 codes, unit scales: no block scaling"
         return (fn, 2.0 * M_TOTAL * N * K, nbytes, "fp8",
-                dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, recipe="1x128 act / 128x128 weight, e4m3fn", seed=seed), None)
+                dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, recipe="1x128 act / 128x128 weight, e4m3fn",
+                     group_sizes=size_tag, seed=seed), None)
     if kind == "fp8c":
         from triton_grouped_gemm_amd.gemm.FP8.m_grouped_gemm_channel_expert import gmm_fp8_act_per_channel_w_per_expert
         gen = torch.Generator(device=dev).manual_seed(seed + 3)
@@ -176,8 +216,20 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
         sb = torch.rand(G * N, device=dev, generator=gen) + 0.5
         fn = lambda: gmm_fp8_act_per_channel_w_per_expert(a, sa, w, sb, sizes, torch.bfloat16)
         nbytes = M_TOTAL * K + 4.0 * M_TOTAL + G * N * K + 4.0 * G * N + 2.0 * M_TOTAL * N
+        build_workload.operands = dict(a=a, sa=sa, w=w, sb=sb, sizes=sizes)
+        c_ref = torch.empty((M_TOTAL, N), device=dev, dtype=torch.bfloat16)
+        sb_rows = sb.view(G, 1, N)
+
+        def vendor_loop():  # one library FP8 GEMM per expert with row-wise scales: the same arithmetic
+            for g, (s0, s1) in enumerate(bounds):
+                if s1 > s0:
+                    c_ref[s0:s1] = torch._scaled_mm(a[s0:s1], w[g].t(), scale_a=sa[s0:s1], scale_b=sb_rows[g], out_dtype=torch.bfloat16)
+        build_workload.vendor_loop = vendor_loop
+        build_workload.vendor_out = c_ref
+        build_workload.vendor_kind = "torch._scaled_mm per group (hipBLASLt), row-wise scales, same operands"
         return (fn, 2.0 * M_TOTAL * N * K, nbytes, "fp8",
-                dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, recipe="per-token x per-channel scales, e4m3fn", seed=seed), None)
+                dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, recipe="per-token x per-channel scales, e4m3fn",
+                     group_sizes=size_tag, seed=seed), None)
     if kind == "fp8ck":
         from triton_grouped_gemm_amd.gemm.FP8.k_grouped_gemm_channel_expert import matmul as k_grouped_fp8
         m_dim, n_dim = K, N
@@ -218,16 +270,82 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
     raise ValueError(name)
 
 
+def time_workload(fn, steps: int, warmup: int, dev):
+    """W untimed launches, then `steps` launches each bracketed by HIP events on the launch stream.
+    Returns (wall ms per step, list of per-launch event times in ms)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream(dev)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for s, e in evs:
+        s.record(stream)
+        fn()
+        e.record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return wall_ms, [s.elapsed_time(e) for s, e in evs]
+
+
+def summarise(name: str, flops: float, nbytes: float, dtype_tag: str, wall_ms: float, kernel_ms, uniform: bool):
+    """(value, unit, roofline dict) of one timed workload."""
+    avg_kernel_ms = sum(kernel_ms) / len(kernel_ms)
+    traffic = None if uniform else MEASURED_TRAFFIC_GB.get(name)  # measured on the Dirichlet draw only
+    traffic = None if traffic is None else round(traffic * 1e9)  # bytes per launch
+    if flops > 0:
+        value = flops / (wall_ms * 1e-3) / 1e12
+        peak = PEAK_TFLOPS["fp8" if dtype_tag == "fp8" else "bf16"]
+        achieved = flops / (avg_kernel_ms * 1e-3) / 1e12
+        roofline = dict(bound="mfma", achieved=round(achieved, 2), peak=peak, unit="TFLOP/s",
+                        frac=round(achieved / peak, 4), traffic=traffic,
+                        min_ms=round(min(kernel_ms), 4), avg_ms=round(avg_kernel_ms, 4),
+                        algorithmic_gbytes=round(nbytes / 1e9, 3))
+        return value, "TFLOP/s", roofline
+    value = nbytes / (wall_ms * 1e-3) / 1e9
+    achieved = nbytes / (avg_kernel_ms * 1e-3) / 1e9
+    roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                    frac=round(achieved / PEAK_HBM_GBS, 4), traffic=traffic,
+                    min_ms=round(min(kernel_ms), 4), avg_ms=round(avg_kernel_ms, 4))
+    return value, "GB/s", roofline
+
+
+def time_vendor_loop(flops: float):
+    """The per-group library-GEMM loop that build_workload left behind, or None (also when the library refuses the call)."""
+    vl = build_workload.vendor_loop
+    if vl is None:
+        return None
+    try:
+        vl()
+        torch.cuda.synchronize()
+        n_v = 3
+        tv = time.perf_counter()
+        for _ in range(n_v):
+            vl()
+        torch.cuda.synchronize()
+    except Exception as exc:  # e.g. a scaling mode this torch / hipBLASLt build does not offer
+        return dict(value=None, unit="TFLOP/s", kind=getattr(build_workload, "vendor_kind", ""), error=str(exc).splitlines()[0][:200])
+    v_ms = (time.perf_counter() - tv) * 1e3 / n_v
+    kind = getattr(build_workload, "vendor_kind", None) or "torch.matmul per group (hipBLASLt), same operands"
+    return dict(value=round(flops / (v_ms * 1e-3) / 1e12, 2), unit="TFLOP/s", ms_per_step=round(v_ms, 4),
+                kind=kind + ", wall time incl. launches")
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="bf16_m_grouped_gateup_nt", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS),
+                    help="default: bf16_m_grouped_gateup_nt, followed by fp8_block_m_grouped under the line's \"fp8\" key")
+    ap.add_argument("--uniform-groups", action="store_true",
+                    help="every group gets M / G = 5120 rows, as in the reference's published tables, instead of the "
+                         "Dirichlet-multinomial draw")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="host-core time budget of the CPU baseline sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-vendor-loop", action="store_true",
-                    help="skip timing the per-group torch.matmul (hipBLASLt) loop over the same operands")
+                    help="skip timing the per-group library GEMM loop (hipBLASLt through torch) over the same operands")
+    ap.add_argument("--no-fp8", action="store_true", help="default run: skip the FP8 block-scaled half")
     ap.add_argument("--zeros", action="store_true",
                     help="M-grouped bf16 workloads only: all-zero operands (diagnostic: shows how far the clock is held down "
                          "by the power the multipliers draw on random data); reported as data=synthetic-zeros")
@@ -246,10 +364,17 @@ def main() -> int:
     _native.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    if (args.zeros or args.num_cu > 0) and WORKLOADS[args.workload][0] != "mg":
+    workload = args.workload or "bf16_m_grouped_gateup_nt"
+    with_fp8 = args.workload is None and not args.no_fp8 and not args.zeros and args.num_cu <= 0
+    kind = WORKLOADS[workload][0]
+    if (args.zeros or args.num_cu > 0) and kind != "mg":
         print("--zeros / --num-cu apply to the bf16_m_grouped_* workloads only", file=sys.stderr)
         return 2
-    fn, flops, nbytes, dtype_tag, config, cpu_sample = build_workload(args.workload, dev, zeros=args.zeros, num_cu=args.num_cu)
+    if args.uniform_groups and kind in ("masked", "quant", "permute", "unpermute"):
+        print("--uniform-groups applies to the M-grouped and K-grouped GEMM workloads", file=sys.stderr)
+        return 2
+    fn, flops, nbytes, dtype_tag, config, cpu_sample = build_workload(workload, dev, zeros=args.zeros, num_cu=args.num_cu,
+                                                                      uniform=args.uniform_groups)
     if args.num_cu > 0:
         config["num_cu"] = args.num_cu
 
@@ -259,54 +384,9 @@ def main() -> int:
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    for _ in range(args.warmup):
-        fn()
-    torch.cuda.synchronize()
-    stream = torch.cuda.current_stream(dev)
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    t0 = time.perf_counter()
-    for s, e in evs:
-        s.record(stream)
-        fn()
-        e.record(stream)
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    kernel_ms = [s.elapsed_time(e) for s, e in evs]
-    avg_kernel_ms = sum(kernel_ms) / len(kernel_ms)
-
-    is_gemm = flops > 0
-    traffic = MEASURED_TRAFFIC_GB.get(args.workload)
-    traffic = None if traffic is None else round(traffic * 1e9)  # bytes per launch
-    if is_gemm:
-        value = flops / (wall_ms * 1e-3) / 1e12
-        peak = PEAK_TFLOPS["fp8" if dtype_tag == "fp8" else "bf16"]
-        achieved = flops / (avg_kernel_ms * 1e-3) / 1e12
-        roofline = dict(bound="mfma", achieved=round(achieved, 2), peak=peak, unit="TFLOP/s",
-                        frac=round(achieved / peak, 4), traffic=traffic,
-                        min_ms=round(min(kernel_ms), 4), avg_ms=round(avg_kernel_ms, 4),
-                        algorithmic_gbytes=round(nbytes / 1e9, 3))
-        metric, unit = "grouped GEMM TFLOP/s (2*M*N*K/time), M-grouped G=128", "TFLOP/s"
-    else:
-        value = nbytes / (wall_ms * 1e-3) / 1e9
-        achieved = nbytes / (avg_kernel_ms * 1e-3) / 1e9
-        roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=PEAK_HBM_GBS, unit="GB/s",
-                        frac=round(achieved / PEAK_HBM_GBS, 4), traffic=traffic,
-                        min_ms=round(min(kernel_ms), 4), avg_ms=round(avg_kernel_ms, 4))
-        metric, unit = "streaming kernel algorithmic GB/s", "GB/s"
-
-    vendor = None
-    if build_workload.vendor_loop is not None and not args.no_vendor_loop:
-        vl = build_workload.vendor_loop
-        vl()
-        torch.cuda.synchronize()
-        n_v = 3
-        tv = time.perf_counter()
-        for _ in range(n_v):
-            vl()
-        torch.cuda.synchronize()
-        v_ms = (time.perf_counter() - tv) * 1e3 / n_v
-        vendor = dict(value=round(flops / (v_ms * 1e-3) / 1e12, 2), unit="TFLOP/s", ms_per_step=round(v_ms, 4),
-                      kind="torch.matmul per group (hipBLASLt), same operands, wall time incl. launches")
+    wall_ms, kernel_ms = time_workload(fn, args.steps, args.warmup, dev)
+    value, unit, roofline = summarise(workload, flops, nbytes, dtype_tag, wall_ms, kernel_ms, args.uniform_groups)
+    vendor = None if args.no_vendor_loop else time_vendor_loop(flops)
 
     cpu_baseline = None
     if cpu_sample is not None and not args.no_cpu_baseline:
@@ -314,12 +394,26 @@ def main() -> int:
         cpu_baseline = dict(value=round(tf, 4), unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
                             sample=sample, host_cpus=os.cpu_count())
 
-    print(json.dumps({
-        "metric": metric, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps,
+    line = {
+        "metric": METRICS[kind], "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dtype_tag, "data": "synthetic-zeros" if args.zeros else "synthetic", "config": config,
         "roofline": roofline, "cpu_baseline": cpu_baseline, "vendor_loop": vendor,
-    }))
+    }
+
+    if with_fp8:  # the FP8 half of the headline metric: same run, same steps and warm-up, its own operands
+        del fn, cpu_sample
+        build_workload.vendor_loop = build_workload.vendor_out = None
+        build_workload.operands = {}
+        torch.cuda.empty_cache()
+        name8 = "fp8_block_m_grouped"
+        fn8, flops8, nbytes8, tag8, config8, _ = build_workload(name8, dev, uniform=args.uniform_groups)
+        wall8, kms8 = time_workload(fn8, args.steps, args.warmup, dev)
+        value8, unit8, roof8 = summarise(name8, flops8, nbytes8, tag8, wall8, kms8, args.uniform_groups)
+        line["fp8"] = {"metric": METRICS["fp8"], "value": round(value8, 2), "unit": unit8, "ms_per_step": round(wall8, 4),
+                       "dtype": tag8, "config": config8, "roofline": roof8,
+                       "vendor_loop": None if args.no_vendor_loop else time_vendor_loop(flops8)}
+    print(json.dumps(line))
     return 0
 
 
