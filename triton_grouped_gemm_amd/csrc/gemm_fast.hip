@@ -191,9 +191,10 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
       io.b_rem = klen;
       io.b_off = t.n0 * 2;
     } else {
-      const int64_t rows_left = p.m_total - t.row0;
+      // only the tile's valid rows are fetched: the rest of its 256 (another group's rows, or whatever lies beyond
+      // masked_m) reads as zero and its products are never stored
       io.a_base = (uint64_t)p.A + (uint64_t)(t.row0 * a_ld);
-      io.a_rem = (int)(rows_left < C::BM ? rows_left : C::BM) * (int)a_ld;
+      io.a_rem = t.rows * (int)a_ld;
       if (LAYOUT == LAYOUT_NT) {
         const int n_left = p.N - t.n0;
         io.b_base = (uint64_t)p.B + (uint64_t)(((int64_t)t.g * p.N + t.n0) * b_ld);

@@ -116,8 +116,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
     TileIo io;
     const int64_t k0 = KGROUP ? t.k0 : 0;
     io.kt_n = __builtin_amdgcn_readfirstlane(slabs_of(t));
-    const int64_t rows_left = p.m_total - t.row0;
-    const int a_rows = (int)(rows_left < C::BM ? rows_left : C::BM);
+    const int a_rows = t.rows;  // only the tile's valid rows are fetched, the others read as zero
     const int n_left = p.N - t.n0;
     io.a_base = uniform64((uint64_t)p.A + (uint64_t)(t.row0 * ld + k0));
     io.a_left = __builtin_amdgcn_readfirstlane((int)((int64_t)a_rows * ld - k0));

@@ -125,9 +125,8 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   const int64_t b_step = B_KMAJOR ? BK4 * 2 : (int64_t)BK4 * b_ld;
   auto make_io = [&](const Tile& t) {
     TileIo io;
-    const int64_t rows_left = p.m_total - t.row0;
     io.a_base = uniform64((uint64_t)p.A + (uint64_t)(t.row0 * a_ld));
-    io.a_rem = __builtin_amdgcn_readfirstlane((int)(rows_left < C::BM ? rows_left : C::BM) * a_ld);
+    io.a_rem = __builtin_amdgcn_readfirstlane(t.rows * a_ld);  // only the tile's valid rows are fetched
     io.b_off = 0;
     if (B_KMAJOR) {
       const int n_left = p.N - t.n0;
