@@ -23,15 +23,19 @@ def _ints(shape, seed, dtype=torch.bfloat16, lo=-1, hi=1):
     return torch.randint(lo, hi + 1, shape, generator=g).to(dtype)
 
 
-@pytest.fixture(params=[0, 1, 2], ids=["tuned", "generic", "four_wave"])
+@pytest.fixture(params=[0, 1, 2, 3], ids=["tuned", "generic", "four_wave", "stream"])
 def variant(request, dev):
     """tuned: what a call gets by default; generic: the shape-agnostic kernel; four_wave: the large-problem kernel
-    forced onto every M-grouped NT shape it can take, whatever the size (other calls run as in `tuned`)."""
+    forced onto every M-grouped NT shape it can take, whatever the size; stream: the weight-streaming configuration
+    (128-row tiles, three B slab buffers) forced onto every M-grouped / masked launch, whatever the group sizes
+    (other calls run as in `tuned`)."""
     _native.set_option("force_generic", int(request.param == 1))
     _native.set_option("four_wave", 2 if request.param == 2 else 0)
+    _native.set_option("variant", 4 if request.param == 3 else 0)
     yield request.param
     _native.set_option("force_generic", 0)
     _native.set_option("four_wave", 0)
+    _native.set_option("variant", 0)
 
 
 def test_config1_tiny_reference_case(dev, variant):
@@ -65,6 +69,21 @@ def test_m_grouped_exact_on_integer_inputs(dev, variant, dtype, trans_b, sizes, 
     out = m_grouped_gemm(a.to(dev), b.to(dev), s.to(dev), trans_b)
     ref = gemm_ref.gmm_fp32(a, b, sizes, trans_b).to(dtype)
     assert torch.equal(out.cpu(), ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("trans_b", [True, False])
+def test_m_grouped_decode_sized_groups(dev, dtype, trans_b):
+    """No group above 128 rows and more narrow tiles than workgroups: the default launch picks the weight-streaming
+    configuration on the device.  Integer inputs, so the result must equal the oracle bit for bit."""
+    sizes = [(37 * g) % 129 for g in range(48)]  # 0 .. 128
+    sizes[5], sizes[6], sizes[47] = 128, 0, 128  # full 128-row groups and an empty one
+    assert max(sizes) == 128 and min(sizes) == 0
+    M, N, K = sum(sizes), 1032, 200              # ragged last column tile, K tail
+    a = _ints((M, K), 11, dtype)
+    b = _ints((48, N, K) if trans_b else (48, K, N), 12, dtype)
+    out = m_grouped_gemm(a.to(dev), b.to(dev), torch.tensor(sizes, dtype=torch.int32, device=dev), trans_b)
+    assert torch.equal(out.cpu(), gemm_ref.gmm_fp32(a, b, sizes, trans_b).to(dtype))
 
 
 @pytest.mark.parametrize("trans_b", [True, False])
@@ -175,6 +194,23 @@ def test_masked_small(dev, variant, trans_b):
         if mm:
             check_16bit_gemm(blk[:mm], refs[g], refs32[g], f"masked g{g}")
         assert torch.equal(blk[mm:], torch.full((m_max - mm, N), -5.0, dtype=torch.bfloat16))
+
+
+def test_masked_decode_sized_counts(dev):
+    """Masked launch whose counts stay at or below 128 with m_max = 512 (decode): the weight-streaming
+    configuration is picked on the device; exact on integer inputs, rows beyond masked_m untouched."""
+    G, m_max, N, K = 40, 512, 1024, 136
+    masked = [(53 * g) % 129 for g in range(G)]
+    masked[3], masked[4] = 128, 0
+    lhs = _ints((G * m_max, K), 21)
+    rhs = _ints((G, N, K), 22)
+    out = torch.full((G * m_max, N), -5.0, dtype=torch.bfloat16, device=dev)
+    m_grouped_gemm_masked(lhs.to(dev), rhs.to(dev), out, torch.tensor(masked, dtype=torch.int32, device=dev), m_max)
+    out = out.cpu().view(G, m_max, N)
+    ref = torch.bmm(lhs.float().view(G, m_max, K), rhs.float().transpose(1, 2)).to(torch.bfloat16)
+    for g, mm in enumerate(masked):
+        assert torch.equal(out[g, :mm], ref[g, :mm]), f"group {g}"
+        assert bool((out[g, mm:] == -5.0).all()), f"group {g}: rows beyond masked_m were written"
 
 
 def test_masked_full_mask_reduces_to_bmm_exact(dev, variant):

@@ -32,6 +32,7 @@
 //     leave as 16-byte stores that cover whole row segments of the wave's columns.
 #include "fast_common.hpp"
 #include "launch.hpp"
+#include <type_traits>
 
 namespace tgg {
 
@@ -62,9 +63,12 @@ template <int DT> TGG_DEV float from16(uint16_t h) {
   return (float)__builtin_bit_cast(_Float16, h);
 }
 
-template <int BM_, int BN_, int WM_, int WN_>
+// BST: slab buffers of the B operand.  2: A and B slabs of a stage sit together, two stages.  3: the A slabs keep
+// two buffers, the B slabs get a ring of three of their own and their copies run a slab further ahead (the
+// weight-streaming configuration, see gemm_fast_body).
+template <int BM_, int BN_, int WM_, int WN_, int BST_ = 2>
 struct FastCfg {
-  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BST = BST_;
   static constexpr int NWAVES = WM * WN;
   static constexpr int THREADS = NWAVES * 64;
   static constexpr int A_BYTES = BM * BK * 2, B_BYTES = BN * BK * 2;
@@ -73,12 +77,16 @@ struct FastCfg {
   static constexpr int TM = BM / WM / 16, TN = BN / WN / 16;  // 16x16 blocks per wave
   static constexpr int EPI_PITCH = TN * 32 + 16;  // staged strip of 16 rows x (16 TN) 16-bit outputs: row pitch in bytes
   static constexpr int EPI_WAVE_BYTES = 16 * EPI_PITCH;
-  static constexpr int SCHED_OFF = 2 * STAGE_BYTES;
+  static constexpr int SCHED_OFF = 2 * A_BYTES + BST * B_BYTES;
+  // byte offsets of A buffer a (0, 1) and B buffer b (0 .. BST-1)
+  static constexpr int a_off(int a) { return BST == 2 ? a * STAGE_BYTES : a * A_BYTES; }
+  static constexpr int b_off(int b) { return BST == 2 ? b * STAGE_BYTES + A_BYTES : 2 * A_BYTES + b * B_BYTES; }
   static constexpr int EPI_OFF = SCHED_OFF + (((int)sizeof(SchedTableT<kFastMaxGroups>) + 255) & ~255);
   static constexpr int QMAX_OFF = EPI_OFF + NWAVES * EPI_WAVE_BYTES;  // fused quantisation: [WN][BM] 16-bit row maxima
   static constexpr int SMEM_BYTES = QMAX_OFF + WN * BM * 2;
   static_assert(NI_A % NWAVES == 0 && NI_B % NWAVES == 0, "copies must divide evenly over waves");
   static_assert(NWAVES % 8 == 0, "a wave keeps one swizzle pattern for all its copies");
+  static_assert(BST == 2 || BST == 3, "B slab buffers");
   static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
 };
 
@@ -88,6 +96,11 @@ template <class C, int DT, int LAYOUT, bool QUANT, int SCHED_AT>
 TGG_DEV void gemm_fast_body(const GemmParams& p) {
   constexpr bool A_KMAJOR = LAYOUT != LAYOUT_TN;
   constexpr bool B_KMAJOR = LAYOUT == LAYOUT_NT;
+  // DEEP: three B slab buffers, B copies one slab further ahead than A copies.  For launches that stream weights
+  // (few rows per group, decode): what limits them is how many bytes of B a CU has in flight, and a B slab of the
+  // two-buffer scheme is requested only one slab period before it is needed.
+  constexpr bool DEEP = C::BST == 3;
+  static_assert(!DEEP || !QUANT, "the fused-quantisation epilogue uses the two-buffer configuration");
   typedef Operand<C::BM, A_KMAJOR> OpA;
   typedef Operand<C::BN, B_KMAJOR> OpB;
 
@@ -153,8 +166,7 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
     const i16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)(q + 4 * (C::BM * 2)));
     return __builtin_bit_cast(i32x4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
-  auto load_b = [&](const char* s, int ks, int j) -> i32x4_t {
-    const char* sb = s + C::A_BYTES;
+  auto load_b = [&](const char* sb, int ks, int j) -> i32x4_t {  // sb: the B slab
     if (B_KMAJOR) return *(const i32x4_t*)(sb + b_rd[ks] + j * 16 * 128);
     const char* q = sb + b_rd[j] + ks * 32 * (C::BN * 2);
     const i16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_ptr_t)q);
@@ -229,13 +241,37 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
   Tile seen;
   int64_t seen_id = -1;
   int seen_g = -1;
+  // DEEP: the B copies have a cursor of their own, one slab ahead of `feed` (which then serves A only); it does
+  // the tile lookups and `feed` reuses them.
+  TileIo feedb;
+  int64_t feedb_id = -1;
+  Tile seenb;
+  int64_t seenb_id = -1;
+  int seenb_g = -1;
+  auto feedb_seek = [&](int64_t id) {
+    feedb.kt_n = 0;
+    feedb.issued = 0;
+    feedb.a_base = feedb.b_base = (uint64_t)p.A;
+    feedb.a_rem = feedb.b_rem = feedb.a_off = feedb.b_off = 0;
+    for (; id < walk.end; id += walk.stride) {
+      const Tile tt = sched_tile<C::BM, C::BN>(p, sched, id, seenb_g);
+      seenb = tt;
+      seenb_id = id;
+      seenb_g = tt.g;
+      if (slabs_of(tt) > 0) {
+        feedb = make_io(tt);
+        break;
+      }
+    }
+    feedb_id = id;
+  };
   auto feed_seek = [&](int64_t id) {
     feed.kt_n = 0;
     feed.issued = 0;
     feed.a_base = feed.b_base = (uint64_t)p.A;
     feed.a_rem = feed.b_rem = feed.a_off = feed.b_off = 0;
     for (; id < walk.end; id += walk.stride) {
-      const Tile tt = sched_tile<C::BM, C::BN>(p, sched, id, seen_g);
+      const Tile tt = (DEEP && id == seenb_id) ? seenb : sched_tile<C::BM, C::BN>(p, sched, id, seen_g);
       seen = tt;
       seen_id = id;
       seen_g = tt.g;
@@ -250,8 +286,8 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
   // begin_slab fixes the descriptors and moves the feed on, copy_k issues this wave's k-th copy.
   struct SlabCopy {
     i32x4_t ra, rb;
-    uint32_t base;
-    bool tail;  // the tile's last slab, cut short by K
+    uint32_t base, base_b;  // LDS addresses of the A slab and of the B slab
+    bool tail, tail_b;      // the tile's last slab, cut short by K (DEEP: A and B are slabs of different numbers)
   };
   constexpr int CA = C::NI_A / C::NWAVES, CB = C::NI_B / C::NWAVES, NC = CA + CB;
   // multiplies between two copies: the first half of a slab's copies goes out right after the barrier, one per
@@ -261,21 +297,39 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
   constexpr int SP2 = (C::TM * C::TN / 2) / (NC / 2);
   constexpr int SP1 = LAYOUT == LAYOUT_TN ? SP2 : 1;
   static_assert(NC % 2 == 0 && SP2 >= 1, "a slab's copies are spread over the multiplies of two half K steps");
-  auto begin_slab = [&](int buf) {
+  // DEEP: the next B slab of the B cursor, into B buffer `buf_b`
+  auto begin_b = [&](SlabCopy& sc, int buf_b) {
+    const bool live = feedb.issued < feedb.kt_n;
+    const int b_len = B_KMAJOR ? feedb.b_rem : min(feedb.b_rem, BK) * (int)b_ld - feedb.b_off;
+    sc.rb = make_rsrc32(feedb.b_base, live ? b_len : 0);
+    sc.base_b = smem_addr + C::b_off(buf_b);
+    sc.tail_b = tail_chunks != 0 && feedb.issued + 1 == feedb.kt_n;
+    feedb.b_base += b_step;
+    feedb.b_rem -= B_KMAJOR ? BK * 2 : BK;
+    feedb.issued += 1;
+    if (live && feedb.issued >= feedb.kt_n) feedb_seek(feedb_id + walk.stride);
+  };
+  // buf: the A buffer (and, with two B buffers, the B buffer); buf_b: the B buffer of the deep ring
+  auto begin_slab = [&](int buf, int buf_b = 0) {
     SlabCopy sc;
     const bool live = feed.issued < feed.kt_n;
     const int a_len = A_KMAJOR ? feed.a_rem : min(feed.a_rem, BK) * (int)a_ld - feed.a_off;
     const int b_len = B_KMAJOR ? feed.b_rem : min(feed.b_rem, BK) * (int)b_ld - feed.b_off;
     sc.ra = make_rsrc32(feed.a_base, live ? a_len : 0);
-    sc.rb = make_rsrc32(feed.b_base, live ? b_len : 0);
-    sc.base = smem_addr + buf * C::STAGE_BYTES;
+    sc.base = smem_addr + C::a_off(buf);
     sc.tail = tail_chunks != 0 && feed.issued + 1 == feed.kt_n;
+    if (!DEEP) {
+      sc.rb = make_rsrc32(feed.b_base, live ? b_len : 0);
+      sc.base_b = sc.base + C::A_BYTES;
+      sc.tail_b = sc.tail;
+    }
     feed.a_base += a_step;
     feed.a_rem -= A_KMAJOR ? BK * 2 : BK;
     feed.b_base += b_step;
     feed.b_rem -= B_KMAJOR ? BK * 2 : BK;
     feed.issued += 1;
     if (live && feed.issued >= feed.kt_n) feed_seek(feed_id + walk.stride);
+    if (DEEP) begin_b(sc, buf_b);
     return sc;
   };
   auto copy_k = [&](const SlabCopy& sc, int k) {
@@ -284,7 +338,7 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
       copy_b128_to_lds(sc.ra, sc.base + idx * 1024, (sc.tail ? a_voff_tail : a_voff) + idx * OpA::RPI * (int)a_ld);
     } else {
       const int idx = wave + (k - CA) * C::NWAVES;
-      copy_b128_to_lds(sc.rb, sc.base + C::A_BYTES + idx * 1024, (sc.tail ? b_voff_tail : b_voff) + idx * OpB::RPI * (int)b_ld);
+      copy_b128_to_lds(sc.rb, sc.base_b + idx * 1024, (sc.tail_b ? b_voff_tail : b_voff) + idx * OpB::RPI * (int)b_ld);
     }
   };
 
@@ -302,24 +356,34 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
   // for.  They are spread out because the texture-address unit takes 16 cycles per copy instruction and its
   // queue is short: a wave that issues its copies back to back sits blocked behind the other waves' copies with
   // its multiplies queued up behind them.  Tile boundaries do not interrupt the stream.
+  // DEEP: per slab r the A copies of slab r+2 and then the B copies of slab r+3 are issued; the wait in slab r+1
+  // lets the most recent CB copies (those B copies) stay in flight: loads complete in order, so all older ones are done.
+  constexpr int WAIT_N = DEEP ? CB : 0;
+  if (DEEP) feedb_seek(walk.first);
   feed_seek(walk.first);
   {
-    const SlabCopy s0 = begin_slab(0);
+    SlabCopy s0 = begin_slab(0, 0);
 #pragma unroll
     for (int k = 0; k < NC; ++k) copy_k(s0, k);
+    if (DEEP) {  // B slab 1 as well: from here on the B cursor is a slab ahead
+      begin_b(s0, 1);
+#pragma unroll
+      for (int k = CA; k < NC; ++k) copy_k(s0, k);
+    }
   }
   wait_vmcnt<0>();
   __syncthreads();
-  SlabCopy sc = begin_slab(1);
+  SlabCopy sc = begin_slab(1, 2);
 #pragma unroll
   for (int k = 0; k < NC / 2; ++k) copy_k(sc, k);
   i32x4_t fa[C::TM - 1], fa_last[2], fb[2][C::TN];
 #pragma unroll
-  for (int i = 0; i < C::TM - 1; ++i) fa[i] = load_a(smem, 0, i);
-  fa_last[0] = load_a(smem, 0, C::TM - 1);
+  for (int i = 0; i < C::TM - 1; ++i) fa[i] = load_a(smem + C::a_off(0), 0, i);
+  fa_last[0] = load_a(smem + C::a_off(0), 0, C::TM - 1);
 #pragma unroll
-  for (int j = 0; j < C::TN; ++j) fb[0][j] = load_b(smem, 0, j);
+  for (int j = 0; j < C::TN; ++j) fb[0][j] = load_b(smem + C::b_off(0), 0, j);
   int ring = 0;
+  int ring3 = 0;  // ring % 3 (DEEP: the B buffer of the current slab)
 
   // The accumulators start at zero and every epilogue path below clears each strip's registers right after it
   // has converted them: those moves then sit in the epilogue's LDS waits instead of in front of the next tile's
@@ -352,7 +416,7 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
     // Copies [k0, k0 + NC/2) of `sc` are issued between the multiplies when k0 >= 0 (SP1, SP2 above).
     enum { READ_EARLY, READ_ROLL, READ_NONE, READ_CATCH_UP };
     SlabCopy sc_next;
-    auto half = [&](int cur_set, int h, const char* s_next, int ks_next, int mode, int k0, bool prepare = false) {
+    auto half = [&](int cur_set, int h, const char* s_next, const char* sb_next, int ks_next, int mode, int k0, bool prepare = false) {
       const int nxt = cur_set ^ 1;
       constexpr int HM = C::TM / 2;
 #pragma unroll
@@ -370,7 +434,7 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
           if (n == 0 && (mode == READ_EARLY || mode == READ_CATCH_UP)) {
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int j2 = 0; j2 < C::TN; ++j2) fb[nxt][j2] = load_b(s_next, ks_next, j2);
+            for (int j2 = 0; j2 < C::TN; ++j2) fb[nxt][j2] = load_b(sb_next, ks_next, j2);
             fa_last[nxt] = load_a(s_next, ks_next, C::TM - 1);
             if (mode == READ_CATCH_UP) {
 #pragma unroll
@@ -378,7 +442,7 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
             }
             __builtin_amdgcn_sched_barrier(0);
           }
-          if (prepare && n == 1) sc_next = begin_slab(ring & 1);  // scalar work, under the multiplies just issued
+          if (prepare && n == 1) sc_next = begin_slab(ring & 1, ring3);  // scalar work, under the multiplies just issued
           const int sp = k0 == 0 ? SP1 : SP2;
           if (k0 >= 0 && (n + 1) % sp == 0 && (n + 1) / sp <= NC / 2) {
             __builtin_amdgcn_sched_barrier(0);
@@ -406,8 +470,8 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
           copy_k(sc, k);
           __builtin_amdgcn_s_sleep(1);  // paced: the address unit's queue is shared with the working waves
         }
-        sc_next = begin_slab(ring & 1);
-        wait_vmcnt<0>();
+        sc_next = begin_slab(ring & 1, ring3);
+        wait_vmcnt<WAIT_N>();
         __syncthreads();
         sc = sc_next;
 #pragma unroll
@@ -416,29 +480,35 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
           __builtin_amdgcn_s_sleep(1);
         }
         ++ring;
+        ring3 = ring3 == 2 ? 0 : ring3 + 1;
       }
       if (kt_n > 0) {
-        const char* sn = smem + (ring & 1) * C::STAGE_BYTES;
+        const char* sn = smem + C::a_off(ring & 1);
+        const char* sbn = smem + C::b_off(DEEP ? ring3 : (ring & 1));
 #pragma unroll
         for (int i = 0; i < C::TM - 1; ++i) fa[i] = load_a(sn, 0, i);
         fa_last[0] = load_a(sn, 0, C::TM - 1);
 #pragma unroll
-        for (int j = 0; j < C::TN; ++j) fb[0][j] = load_b(sn, 0, j);
+        for (int j = 0; j < C::TN; ++j) fb[0][j] = load_b(sbn, 0, j);
       }
       continue;
     }
 
     for (int kt = 0; kt < kt_n; ++kt) {
-      const char* sa = smem + (ring & 1) * C::STAGE_BYTES;
-      const char* sn = smem + ((ring + 1) & 1) * C::STAGE_BYTES;
-      half(0, 0, sa, 1, READ_EARLY, NC / 2);
-      half(0, 1, sa, 1, READ_ROLL, -1, true);
-      half(1, 0, sn, 0, READ_NONE, -1);
-      wait_vmcnt<0>();
+      const int ring3n = ring3 == 2 ? 0 : ring3 + 1;
+      const char* sa = smem + C::a_off(ring & 1);
+      const char* sn = smem + C::a_off((ring + 1) & 1);
+      const char* sba = smem + C::b_off(DEEP ? ring3 : (ring & 1));
+      const char* sbn = smem + C::b_off(DEEP ? ring3n : ((ring + 1) & 1));
+      half(0, 0, sa, sba, 1, READ_EARLY, NC / 2);
+      half(0, 1, sa, sba, 1, READ_ROLL, -1, true);
+      half(1, 0, sn, sbn, 0, READ_NONE, -1);
+      wait_vmcnt<WAIT_N>();
       __syncthreads();
       sc = sc_next;
-      half(1, 1, sn, 0, READ_CATCH_UP, 0);
+      half(1, 1, sn, sbn, 0, READ_CATCH_UP, 0);
       ++ring;
+      ring3 = ring3n;
     }
 
     // Epilogue.  A lane owns row l16 and columns 16 j + 4 lg + (0..3) of each 16-row block i: transpose one
@@ -572,22 +642,42 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
   gemm_fast_body<C, DT, LAYOUT, QUANT, C::SCHED_OFF>(p);
 }
 
-// Two tile configurations in one kernel, chosen per launch from the group sizes, which only the device knows:
-// the narrow tiles (half the columns) when all of them fit into a single round of the persistent workgroups
-// -- twice as many workgroups then have work, and a narrow tile costs about 0.7 of a wide one -- and the wide
-// tiles otherwise.  Both use BM-row tiles, so one group table serves both; it sits where the wide configuration
-// keeps it, past everything the narrow one touches.
-template <class CW, class CN, int DT, int LAYOUT>
+// Several tile configurations in one kernel, chosen per launch from the group sizes, which only the device knows:
+//   * the narrow tiles (half the columns) when all of them fit into a single round of the persistent workgroups
+//     -- twice as many workgroups then have work, and a narrow tile costs about 0.7 of a wide one;
+//   * otherwise, when no group has more than 128 rows (decode-sized groups: the launch streams weights), the
+//     weight-streaming configuration CS -- 128-row tiles and a ring of three B slabs whose copies run a slab
+//     further ahead, i.e. twice the weight bytes in flight per CU: 5-15 % faster there (up to 6 TB/s of weights);
+//   * the wide tiles otherwise.
+// Wide and narrow use BM-row tiles, so one group table serves both; with at most 128 rows per group every group
+// has at most one row tile of either height, so the same table serves CS too.  It sits where the wide configuration
+// keeps it, past everything the others touch.  CS = void: no weight-streaming configuration (K-grouped).
+template <class CW, class CN, class CS, int DT, int LAYOUT>
 __global__ __launch_bounds__(CW::THREADS) void gemm_fast_auto_kernel(const GemmParams p) {
   static_assert(CW::BM == CN::BM && CW::THREADS == CN::THREADS, "one group table, one launch shape");
   static_assert(CN::SMEM_BYTES <= CW::SCHED_OFF, "the narrow configuration must not reach the shared group table");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + CW::SCHED_OFF);
   sched_init<CW::BM>(p, sched);
-  if (__builtin_expect(sched_num_tiles<CN::BM, CN::BN>(p, sched) > (int64_t)gridDim.x, 1))
+  bool stream = false;
+  if constexpr (!std::is_void<CS>::value) {
+    static_assert(CS::THREADS == CW::THREADS && CS::SCHED_OFF == CW::SCHED_OFF && CS::SMEM_BYTES <= CW::SMEM_BYTES,
+                  "the weight-streaming configuration shares the launch shape and the group table's place");
+    static_assert(CW::THREADS >= kFastMaxGroups, "one group per thread in the test below");
+    const int big = (int)threadIdx.x < p.G && sched.rows[threadIdx.x] > CS::BM;
+    stream = __syncthreads_or(big) == 0;
+  }
+  if (__builtin_expect(sched_num_tiles<CN::BM, CN::BN>(p, sched) > (int64_t)gridDim.x, 1)) {
+    if constexpr (!std::is_void<CS>::value) {
+      if (__builtin_expect(stream, 0)) {
+        gemm_fast_body<CS, DT, LAYOUT, false, CW::SCHED_OFF>(p);
+        return;
+      }
+    }
     gemm_fast_body<CW, DT, LAYOUT, false, CW::SCHED_OFF>(p);
-  else
+  } else {
     gemm_fast_body<CN, DT, LAYOUT, false, CW::SCHED_OFF>(p);
+  }
 }
 
 template <class Kern>
@@ -621,10 +711,10 @@ int launch_cfg(const GemmParams& p, hipStream_t s) {
   return launch_kernel(gemm_fast_kernel<C, DT, LAYOUT, QUANT>, C::SMEM_BYTES, C::THREADS, attr_flag(attr_set), p, s, "gemm_fast");
 }
 
-template <class CW, class CN, int DT, int LAYOUT>
+template <class CW, class CN, class CS, int DT, int LAYOUT>
 int launch_auto(const GemmParams& p, hipStream_t s) {
   static bool attr_set[64] = {false};
-  return launch_kernel(gemm_fast_auto_kernel<CW, CN, DT, LAYOUT>, CW::SMEM_BYTES, CW::THREADS, attr_flag(attr_set), p, s, "gemm_fast");
+  return launch_kernel(gemm_fast_auto_kernel<CW, CN, CS, DT, LAYOUT>, CW::SMEM_BYTES, CW::THREADS, attr_flag(attr_set), p, s, "gemm_fast");
 }
 
 int g_variant = 0;
@@ -633,11 +723,16 @@ template <int DT, int LAYOUT>
 int launch_variant(const GemmParams& p, hipStream_t s) {
   typedef FastCfg<256, 256, 2, 4> Wide;
   typedef FastCfg<256, 128, 2, 4> Narrow;
+  typedef FastCfg<128, 256, 2, 4, 3> Stream;
+  typedef typename std::conditional<LAYOUT == LAYOUT_TN, void, Stream>::type StreamOrNone;
   switch (g_variant) {
     default:
-    case 0: return launch_auto<Wide, Narrow, DT, LAYOUT>(p, s);
+    case 0: return launch_auto<Wide, Narrow, StreamOrNone, DT, LAYOUT>(p, s);
     case 1: return launch_cfg<Narrow, DT, LAYOUT, false>(p, s);
     case 2: return launch_cfg<Wide, DT, LAYOUT, false>(p, s);
+    case 4:
+      if constexpr (LAYOUT != LAYOUT_TN) return launch_cfg<Stream, DT, LAYOUT, false>(p, s);
+      else return launch_auto<Wide, Narrow, void, DT, LAYOUT>(p, s);
   }
 }
 
