@@ -1,0 +1,100 @@
+"""Wait-state hazards around the inline-assembly memory instructions of the HIP kernels.
+
+The compiler inserts the wait states gfx9-family hardware needs between certain instruction pairs, but it does not
+look inside inline assembly.  Two of those pairs involve the hand-written vector-memory instructions of the tuned
+kernels (direct-to-LDS copies, non-temporal stores):
+  * a vector instruction writes a scalar register (v_readlane / v_readfirstlane, e.g. the reload of a spilled scalar)
+    and a vector-memory instruction reads that register fewer than five wait states later: it sees the old value --
+    for a buffer descriptor that means a wild address;
+  * a 12- or 16-byte store is followed within two wait states by a vector instruction that overwrites its data
+    registers: the store writes the new value.
+Both were met while developing these kernels (a GPU memory fault, and wrong dwords in the output).  The build keeps
+the device assembly (triton_grouped_gemm_amd/build/*.gfx950.s); this test scans it.  The scanner itself is checked
+on hand-written snippets, so the file tests something even where the library has not been built.
+"""
+import re
+from pathlib import Path
+
+import pytest
+
+BUILD = Path(__file__).resolve().parents[1] / "triton_grouped_gemm_amd" / "build"
+
+
+def _regs(tok: str, kind: str):
+    m = re.match(kind + r"\[(\d+):(\d+)\]$", tok)
+    if m:
+        return set(range(int(m.group(1)), int(m.group(2)) + 1))
+    m = re.match(kind + r"(\d+)$", tok)
+    return {int(m.group(1))} if m else set()
+
+
+def _wait_states(line: str) -> int:
+    m = re.match(r"s_nop (\d+)", line)
+    return int(m.group(1)) + 1 if m else 1
+
+
+def scan(text: str):
+    """Returns a list of (first instruction, second instruction, wait states between them) for every hazard found."""
+    code = []
+    for raw in text.splitlines():
+        line = raw.split(";")[0].strip()
+        if line and not line.startswith(".") and not line.endswith(":"):
+            code.append(line)
+    bad = []
+    for i, line in enumerate(code):
+        op = line.split()[0]
+        toks = [t.strip(",") for t in line.split()[1:]]
+        if not op.startswith(("buffer_", "global_", "flat_", "scratch_")):
+            continue
+        need = set().union(*[_regs(t, "s") for t in toks]) if toks else set()
+        ws = 0
+        for d in range(1, 8):
+            if not need or i - d < 0 or ws >= 5:
+                break
+            prev = code[i - d]
+            ptoks = prev.split()
+            if ptoks[0].startswith("v_") and len(ptoks) > 1 and _regs(ptoks[1].strip(","), "s") & need:
+                bad.append((prev, line, ws))
+                break
+            ws += _wait_states(prev)
+        if re.match(r"(buffer|global|flat|scratch)_store_dwordx[34]", op):
+            data = _regs(toks[0], "v") if op.startswith("buffer") else _regs(toks[1], "v")
+            ws = 0
+            for d in range(1, 4):
+                if i + d >= len(code) or ws >= 2:
+                    break
+                nxt = code[i + d]
+                ntoks = nxt.split()
+                if ntoks[0].startswith("v_") and len(ntoks) > 1 and _regs(ntoks[1].strip(","), "v") & data:
+                    bad.append((line, nxt, ws))
+                    break
+                ws += _wait_states(nxt)
+    return bad
+
+
+def test_scanner_finds_scalar_write_before_vector_memory_read():
+    hazard = "v_readlane_b32 s47, v254, 19\ns_waitcnt lgkmcnt(0)\nbuffer_store_dwordx4 v[2:5], v6, s[44:47], 0 offen nt\n"
+    assert len(scan(hazard)) == 1
+    spaced = "v_readlane_b32 s47, v254, 19\ns_nop 4\nbuffer_store_dwordx4 v[2:5], v6, s[44:47], 0 offen nt\ns_nop 1\n"
+    assert scan(spaced) == []
+    other_register = "v_readlane_b32 s12, v254, 19\nbuffer_load_dwordx4 v1, s[44:47], 0 offen lds\n"
+    assert scan(other_register) == []
+    scalar_writer = "s_mov_b32 s44, s3\nbuffer_load_dwordx4 v1, s[44:47], 0 offen lds\n"  # scalar writes are interlocked
+    assert scan(scalar_writer) == []
+
+
+def test_scanner_finds_overwritten_store_data():
+    hazard = "global_store_dwordx4 v[8:9], v[0:3], off nt\nv_add_u32_e32 v0, 64, v8\n"
+    assert len(scan(hazard)) == 1
+    assert scan("global_store_dwordx4 v[8:9], v[0:3], off nt\ns_nop 1\nv_add_u32_e32 v0, 64, v8\n") == []
+    assert scan("global_store_dwordx4 v[8:9], v[0:3], off nt\nv_add_u32_e32 v12, 64, v8\nv_mov_b32_e32 v13, v1\nv_mov_b32_e32 v0, v1\n") == []
+    assert scan("global_store_dwordx2 v[8:9], v[0:1], off\nv_add_u32_e32 v0, 64, v8\n") == []  # 8-byte stores are not affected
+
+
+def test_built_kernels_have_no_unspaced_hazard():
+    files = sorted(BUILD.glob("*.gfx950.s"))
+    if not files:
+        pytest.skip("no device assembly in the build directory (the library was built elsewhere or not yet)")
+    for f in files:
+        found = scan(f.read_text())
+        assert not found, f"{f.name}: {len(found)} hazards, first: {found[0]}"

@@ -48,7 +48,17 @@ def build_library(verbose: bool = False, jobs: int | None = None) -> Path:
 
     def compile_one(pair):
         src, obj = pair
-        msg = _run([hipcc, *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)])
+        # -save-temps=obj leaves the intermediate files next to the object; only the device assembly is kept
+        # (build/<stem>.gfx950.s): tests/test_isa_hazards.py reads it to check what the compiler cannot check
+        # around the inline-assembly memory instructions.
+        msg = _run([hipcc, *HIPCC_FLAGS, "-save-temps=obj", "-c", str(src), "-o", str(obj)])
+        for tmp in obj_dir.glob(src.stem + "*"):
+            if tmp == obj:
+                continue
+            if tmp.name == f"{src.stem}-hip-amdgcn-amd-amdhsa-{ARCH}.s":
+                os.replace(tmp, obj_dir / f"{src.stem}.{ARCH}.s")
+            elif tmp.suffix != ".s" or "-" in tmp.name:
+                tmp.unlink()
         if verbose and msg.strip():
             print(msg, file=sys.stderr)
 

@@ -32,7 +32,9 @@ TGG_DEV void copy_b128_to_lds(i32x4_t rsrc, uint32_t lds_addr, int voff) {
 // other CUs of the XCD keep re-reading from L2 (+4 % on a store-heavy shape, K = 768).  The bit is set through
 // the instruction text: the compiler's non-temporal store builtin did not have that effect here.
 TGG_DEV void store_c(i32x4_t* dst, i32x4_t v, int nt) {
-  if (nt) asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(dst), "v"(v) : "memory");
+  // s_nop 1: a vector instruction that overwrites the data registers of a 16-byte store within two wait states
+  // corrupts what is stored, and the compiler, which considers them free after this statement, does not look inside it.
+  if (nt) asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" : : "v"(dst), "v"(v) : "memory");
   else *(__attribute__((address_space(1))) i32x4_t*)(uint64_t)dst = v;
 }
 
