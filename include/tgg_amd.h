@@ -40,6 +40,14 @@ int tgg_m_grouped_gemm(const void* A, const void* B, void* C, const void* sizes,
 int tgg_m_grouped_gemm_padded(const void* A, const void* B, void* C, const void* sizes, int sizes_i64, int G,
                               int64_t M, int N, int K, int align, int dtype, int num_cu, void* stream);
 
+/* As tgg_m_grouped_gemm_padded, but group g's rows are [row_start[g], row_start[g] + sizes[g]): the groups'
+ * regions may lie in any order (they must not overlap; a group has one region).  What a per-row grouped_layout
+ * that lists experts out of ascending order describes; the reference forwards any such layout to its backend
+ * (gemm/deep_gemm_ops.py:24-57). */
+int tgg_m_grouped_gemm_placed(const void* A, const void* B, void* C, const void* sizes, int sizes_i64,
+                              const int32_t* row_start, int G, int64_t M, int N, int K, int dtype, int num_cu,
+                              void* stream);
+
 /* For each g and r < masked_m[g]: C[g*m_stride + r,:] = A[g*m_stride + r,:] . B[g]^T (trans_b=1, B [G,N,K]) or
  * . B[g] (trans_b=0, B [G,K,N]); other rows untouched.  Replaces m_grouped_gemm_masked
  * (gemm/BF16/m_grouped_gemm_masked_TMA.py:164-250); m_stride is its expected_m. */
@@ -75,6 +83,12 @@ int tgg_k_grouped_gemm_fp8_channel(const void* x, const float* xs, const void* y
 int tgg_m_grouped_gemm_fp8_block(const void* Aq, const float* sa, const void* Bq, const float* sb, void* C,
                                  const void* sizes, int sizes_i64, int G, int64_t M, int N, int K, int align,
                                  int sa_mn_major, int num_cu, void* stream);
+
+/* As tgg_m_grouped_gemm_fp8_block with group g's rows at [row_start[g], row_start[g] + sizes[g]), regions in any
+ * order (gemm/deep_gemm_ops.py:60-100 forwards any per-row layout). */
+int tgg_m_grouped_gemm_fp8_block_placed(const void* Aq, const float* sa, const void* Bq, const float* sb, void* C,
+                                        const void* sizes, int sizes_i64, const int32_t* row_start, int G, int64_t M,
+                                        int N, int K, int sa_mn_major, int num_cu, void* stream);
 
 /* bf16 x [M,N] -> codes [N,M_expand] (transposed, each group padded to 128 columns, zero tail) and
  * scales [N/128, M_expand/128].  Replaces trans_per_block_quant_expand_128x

@@ -173,6 +173,38 @@ def test_contiguous_padded_bf16_explicit_layout(dev, psum):
         start += p
 
 
+def _shuffled_layout(sizes, order, block_m=128):
+    """Per-row layout with the experts' padded regions laid down in `order`; returns (layout, start row per expert)."""
+    lay, starts, pos = [], {}, 0
+    for g in order:
+        padded = (sizes[g] + block_m - 1) // block_m * block_m
+        starts[g] = pos
+        lay += [g] * sizes[g] + [-1] * (padded - sizes[g])
+        pos += padded
+    return torch.tensor(lay, dtype=torch.int32), starts
+
+
+@pytest.mark.parametrize("layout_dtype", [torch.int32, torch.int64])
+def test_contiguous_bf16_per_row_layout_in_any_expert_order(dev, variant, layout_dtype):
+    """The reference forwards whatever per-row layout it is given (gemm/deep_gemm_ops.py:24-57): here the experts'
+    regions follow one another in a shuffled order.  Checked row by row from the layout's definition
+    (out[r] = a[r] . b[layout[r]]^T where layout[r] >= 0), integer inputs, bit for bit."""
+    sizes = [100, 0, 128, 300, 7, 256]
+    order = [3, 0, 5, 1, 4, 2]
+    lay, _ = _shuffled_layout(sizes, order)
+    Mp, N, K = lay.numel(), 264, 136
+    a = _ints((Mp, K), 31)
+    b = _ints((len(sizes), N, K), 32)
+    out = torch.full((Mp, N), 3.0, dtype=torch.bfloat16, device=dev)
+    m_grouped_bf16_nt_contiguous(a.to(dev), b.to(dev), torch.tensor(sizes, dtype=torch.int32, device=dev), out=out,
+                                 grouped_layout=lay.to(layout_dtype).to(dev))
+    out = out.cpu()
+    valid = lay >= 0
+    ref = torch.einsum("rk,rnk->rn", a[valid].float(), b[lay[valid].long()].float()).to(torch.bfloat16)
+    assert torch.equal(out[valid], ref)
+    assert bool((out[~valid] == 3.0).all()), "padding rows were written"
+
+
 @pytest.mark.parametrize("trans_b", [True, False])
 def test_masked_small(dev, variant, trans_b):
     G, m_max, N, K = 6, 256, 264, 192

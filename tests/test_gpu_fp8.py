@@ -242,6 +242,35 @@ def test_fp8_block_scaled_exact_with_power_of_two_scales(dev, variant, K):
         start += p
 
 
+def test_fp8_block_scaled_per_row_layout_in_any_expert_order(dev, variant):
+    """Experts' regions in a shuffled order, stated by a per-row layout (gemm/deep_gemm_ops.py:60-100 forwards any):
+    small-integer codes and power-of-two scales, so the closed form is exact; checked row by row from the layout."""
+    g = torch.Generator().manual_seed(71)
+    sizes, order, K, N = [100, 128, 0, 300, 28], [3, 1, 4, 0, 2], 384, 256
+    lay = []
+    for e in order:
+        lay += [e] * sizes[e] + [-1] * ((sizes[e] + 127) // 128 * 128 - sizes[e])
+    lay = torch.tensor(lay, dtype=torch.int32)
+    Mp, G, kb = lay.numel(), len(sizes), K // 128
+    aq = torch.randint(-3, 4, (Mp, K), generator=g).float()
+    bq = torch.randint(-3, 4, (G, N, K), generator=g).float()
+    pw = torch.tensor([0.25, 0.5, 1.0, 2.0])
+    sa = pw[torch.randint(0, 4, (Mp, kb), generator=g)]
+    sb = pw[torch.randint(0, 4, (G, N // 128, kb), generator=g)]
+    out = torch.full((Mp, N), 9.0, dtype=torch.bfloat16, device=dev)
+    m_grouped_fp8_nt_contiguous((aq.to(torch.float8_e4m3fn).to(dev), sa.to(dev)),
+                                (bq.to(torch.float8_e4m3fn).to(dev), sb.to(dev)),
+                                torch.tensor(sizes, dtype=torch.int32, device=dev), out=out, grouped_layout=lay.to(dev))
+    out = out.cpu()
+    valid = lay >= 0
+    e = lay[valid].long()
+    ad = (aq * sa.repeat_interleave(128, dim=1))[valid]                                         # dequantised rows
+    wd = bq * sb.repeat_interleave(128, dim=1).repeat_interleave(128, dim=2)                    # dequantised weights
+    ref = torch.einsum("rk,rnk->rn", ad, wd[e]).to(torch.bfloat16)                              # exact in fp32 here
+    assert torch.equal(out[valid], ref)
+    assert bool((out[~valid] == 9.0).all()), "padding rows were written"
+
+
 def test_fp8_matrix_instruction_truncates_products_below_2_to_minus_13_of_the_largest(dev, variant):
     """Characterisation of gfx950's FP8 MFMA that the FP8 tolerances rest on: within one instruction the products
     are aligned to the largest one and bits below 2^-13 of it are dropped (truncated, not rounded), while the

@@ -88,6 +88,19 @@ def test_sizes_from_explicit_layouts():
         assert sizes_from_layout(rows.to(torch.int64), len(sizes), block_m, False).dtype == torch.int32
 
 
+def test_placement_from_per_row_layout_in_any_expert_order():
+    # a per-row layout whose experts are not in ascending order: rows per expert and their first row, by hand
+    from triton_grouped_gemm_amd.gemm.deep_gemm_ops import placement_from_layout
+    lay = torch.tensor([2, 2, 2, -1, 0, 0, -1, -1, 3, -1, -1, -1], dtype=torch.int32)  # block_m = 4; expert 1 absent
+    rows, first = placement_from_layout(lay, 4)
+    assert rows.tolist() == [2, 0, 3, 1] and first.tolist() == [4, 0, 0, 8]
+    assert rows.dtype == torch.int32 and first.dtype == torch.int32
+    # ascending layouts give the padded starts the builders use
+    sizes = [128, 1, 127, 256, 0]
+    rows, first = placement_from_layout(L.make_deep_gemm_grouped_layout(sizes), len(sizes))
+    assert rows.tolist() == sizes and first.tolist() == [0, 128, 256, 384, 0]
+
+
 def test_reference_named_helpers():
     """gemm/BF16/utils.py of the reference: the per-group torch loop, the group-size draw and the two checks."""
     import random

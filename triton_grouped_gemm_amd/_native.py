@@ -22,11 +22,13 @@ _P, _I, _L = c_void_p, c_int, c_int64
 SIGNATURES = {
     "tgg_m_grouped_gemm": [_P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _I, _P],
     "tgg_m_grouped_gemm_padded": [_P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _I, _P],
+    "tgg_m_grouped_gemm_placed": [_P, _P, _P, _P, _I, _P, _I, _L, _I, _I, _I, _I, _P],
     "tgg_m_grouped_gemm_masked": [_P, _P, _P, _P, _I, _I, _L, _L, _I, _I, _I, _I, _I, _P],
     "tgg_k_grouped_gemm": [_P, _P, _P, _P, _P, _I, _I, _I, _L, _I, _I, _P],
     "tgg_m_grouped_gemm_fp8_channel": [_P, _P, _P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _I, _I, _P],
     "tgg_k_grouped_gemm_fp8_channel": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _L, _I, _I, _I, _P],
     "tgg_m_grouped_gemm_fp8_block": [_P, _P, _P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _I, _P],
+    "tgg_m_grouped_gemm_fp8_block_placed": [_P, _P, _P, _P, _P, _P, _I, _P, _I, _L, _I, _I, _I, _I, _P],
     "tgg_trans_per_block_quant_expand_128x": [_P, _P, _P, _P, _I, _I, _L, _I, _L, _I, _P],
     "tgg_per_token_cast_to_fp8": [_P, _P, _P, _L, _I, _I, _I, _P],
     "tgg_per_block_cast_to_fp8": [_P, _P, _P, _I, _I, _I, _I, _P],

@@ -182,6 +182,24 @@ int tgg_m_grouped_gemm_padded(const void* A, const void* B, void* C, const void*
   return dispatch_16bit(p, dtype, 0, (hipStream_t)stream);
 }
 
+int tgg_m_grouped_gemm_placed(const void* A, const void* B, void* C, const void* sizes, int sizes_i64,
+                              const int32_t* row_start, int G, int64_t M, int N, int K, int dtype, int num_cu,
+                              void* stream) {
+  if (int e = check_common(A, B, C, sizes, G, N)) return e;
+  if (!row_start) return set_error("null row_start pointer");
+  if (M < 0 || K < 0) return set_error("negative M or K");
+  if (M >= (1ll << 31)) return set_error("M=%lld does not fit 32-bit row starts", (long long)M);
+  if (dtype != TGG_BF16 && dtype != TGG_F16) return set_error("data type code %d not supported", dtype);
+  if ((K & 7) || (N & 7)) return set_error("N and K must be multiples of 8 (16-byte rows), got N=%d K=%d", N, K);
+  if (M == 0) return 0;
+  GemmParams p = zero_params();
+  p.A = A; p.B = B; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
+  p.mode = MODE_MG_PAD; p.align = 1; p.row_start = row_start; p.m_total = M; p.N = N; p.K = K;
+  p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K; p.b_sn = K; p.b_sk = 1;
+  p.grid_limit = num_cu;
+  return dispatch_16bit(p, dtype, 0, (hipStream_t)stream);
+}
+
 int tgg_m_grouped_gemm_masked(const void* A, const void* B, void* C, const void* masked_m, int masked_i64, int G,
                               int64_t m_stride, int64_t M, int N, int K, int trans_b, int dtype, int num_cu,
                               void* stream) {
@@ -260,13 +278,14 @@ int tgg_k_grouped_gemm_fp8_channel(const void* x, const float* xs, const void* y
   return launch_generic_fp8_channel(p, fmt_a, fmt_b, TGG_BF16, (hipStream_t)stream);
 }
 
-int tgg_m_grouped_gemm_fp8_block(const void* Aq, const float* sa, const void* Bq, const float* sb, void* C,
-                                 const void* sizes, int sizes_i64, int G, int64_t M, int N, int K, int align,
-                                 int sa_mn_major, int num_cu, void* stream) {
+static int fp8_block_impl(const void* Aq, const float* sa, const void* Bq, const float* sb, void* C, const void* sizes,
+                          int sizes_i64, const int32_t* row_start, int G, int64_t M, int N, int K, int align,
+                          int sa_mn_major, int num_cu, void* stream) {
   if (int e = check_common(Aq, Bq, C, sizes, G, N)) return e;
   if (!sa || !sb) return set_error("null scale pointer");
   if (M < 0 || K < 0) return set_error("negative M or K");
-  if (align < 1 || (align & 127)) return set_error("alignment must be a positive multiple of 128, got %d", align);
+  if (row_start && M >= (1ll << 31)) return set_error("M=%lld does not fit 32-bit row starts", (long long)M);
+  if (!row_start && (align < 1 || (align & 127))) return set_error("alignment must be a positive multiple of 128, got %d", align);
   if (K & 15) return set_error("K must be a multiple of 16 for fp8 operands, got %d", K);
   if (M == 0) return 0;
   GemmParams p = zero_params();
@@ -274,12 +293,25 @@ int tgg_m_grouped_gemm_fp8_block(const void* Aq, const float* sa, const void* Bq
   p.sa = sa; p.sb = sb;
   const int kblocks = (K + 127) / 128;
   if (sa_mn_major) { p.sa_rs = 1; p.sa_ks = M; } else { p.sa_rs = kblocks; p.sa_ks = 1; }
-  p.mode = MODE_MG_PAD; p.align = align; p.m_total = M; p.N = N; p.K = K;
+  p.mode = MODE_MG_PAD; p.align = row_start ? 1 : align; p.row_start = row_start; p.m_total = M; p.N = N; p.K = K;
   p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K; p.b_sn = K; p.b_sk = 1;
   p.grid_limit = num_cu;
   if (!g_force_generic && sa_mn_major && kblocks <= 64 && fast_fp8_supported(p, true))
     return launch_fast_fp8_block(p, (hipStream_t)stream);
   return launch_generic_fp8_block(p, (hipStream_t)stream);
+}
+
+int tgg_m_grouped_gemm_fp8_block(const void* Aq, const float* sa, const void* Bq, const float* sb, void* C,
+                                 const void* sizes, int sizes_i64, int G, int64_t M, int N, int K, int align,
+                                 int sa_mn_major, int num_cu, void* stream) {
+  return fp8_block_impl(Aq, sa, Bq, sb, C, sizes, sizes_i64, nullptr, G, M, N, K, align, sa_mn_major, num_cu, stream);
+}
+
+int tgg_m_grouped_gemm_fp8_block_placed(const void* Aq, const float* sa, const void* Bq, const float* sb, void* C,
+                                        const void* sizes, int sizes_i64, const int32_t* row_start, int G, int64_t M,
+                                        int N, int K, int sa_mn_major, int num_cu, void* stream) {
+  if (!row_start) return set_error("null row_start pointer");
+  return fp8_block_impl(Aq, sa, Bq, sb, C, sizes, sizes_i64, row_start, G, M, N, K, 128, sa_mn_major, num_cu, stream);
 }
 
 int tgg_trans_per_block_quant_expand_128x(const void* x, void* codes, float* scales, const void* sizes,

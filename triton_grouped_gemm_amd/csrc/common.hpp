@@ -75,6 +75,7 @@ struct GemmParams {
   const void* sizes;      // per-group row counts / masked_m / token counts (int32 or int64)
   const int32_t* k_start; // MODE_KG only
   const int32_t* k_end;   // MODE_KG only
+  const int32_t* row_start; // MODE_MG_PAD, optional: group g's rows start at row_start[g] (groups placed in any order)
   const float* scale_m;   // per-row scale (channel modes) or nullptr
   const float* scale_n;   // per-(group, column) scale, indexed g*N + n, or nullptr
   const float* sa;        // block-scaled activation scales: element (row, kb) at row * sa_rs + kb * sa_ks

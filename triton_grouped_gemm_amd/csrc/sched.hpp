@@ -65,7 +65,7 @@ TGG_HD void sched_prefix(const GemmParams& p, Table& t) {
       start = (int64_t)g * p.m_stride;
       if (sz > p.m_stride) sz = p.m_stride;
     } else {
-      start = row;
+      start = (p.mode == MODE_MG_PAD && p.row_start) ? (int64_t)p.row_start[g] : row;
       row += (p.mode == MODE_MG_PAD) ? ((sz + p.align - 1) / p.align) * p.align : sz;
     }
     const int64_t limit = (p.mode == MODE_KG_COUNT) ? p.k_total : p.m_total;

@@ -10,11 +10,12 @@ written.
 ``grouped_layout`` is what the reference forwards to ``deep_gemm``.  When the caller leaves it out it is
 implied by ``size_per_group`` and ``block_m`` (the reference builds it from them).  When the caller passes
 one, the valid rows of every expert are taken from it, on the device and without a host round trip:
-the per-row form ``[M_padded]`` (expert id per row, -1 on padding rows) is counted per expert, the psum form
-``[G]`` (``use_psum_layout=True``: end offset of every expert's valid rows, starts aligned up to ``block_m``)
-is differenced.  Both forms place expert g after expert g-1, each at the next multiple of ``block_m``, as
-``make_deep_gemm_grouped_layout`` / ``make_deep_gemm_psum_layout`` build them; a per-row layout that lists
-experts out of ascending order is not supported.
+the psum form ``[G]`` (``use_psum_layout=True``: end offset of every expert's valid rows, starts aligned up to
+``block_m``) is differenced -- it places expert g after expert g-1 by construction; of the per-row form
+``[M_padded]`` (expert id per row, -1 on padding rows) the rows of every expert are counted and their first row
+is located, so the experts' regions may follow one another in any order (``make_deep_gemm_grouped_layout``
+builds them ascending; a router that fills the buffer in arrival order does not).  One restriction remains: an
+expert's valid rows must be contiguous (one region per expert).
 """
 from __future__ import annotations
 
@@ -66,6 +67,21 @@ def sizes_from_layout(grouped_layout: torch.Tensor, num_groups: int, block_m: in
     return counts[1:].to(torch.int32)
 
 
+def placement_from_layout(grouped_layout: torch.Tensor, num_groups: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-row layout ``[M_padded]`` (expert id per row, -1 = padding) -> ``(rows, first_row)``, both int32 ``[G]``
+    on the layout's device, computed without a host round trip: how many rows carry expert id g and the smallest
+    such row index (0 for experts without rows).  Reference contract: gemm/layout.py:73-97 builds such layouts in
+    ascending expert order, gemm/deep_gemm_ops.py:24-100 forwards whatever the caller passes."""
+    lay = grouped_layout.to(torch.int64)
+    m = lay.shape[0]
+    counts = torch.zeros(num_groups + 1, dtype=torch.int64, device=lay.device)
+    counts.scatter_add_(0, lay + 1, torch.ones_like(lay))
+    first = torch.full((num_groups + 1,), m, dtype=torch.int64, device=lay.device)
+    first.scatter_reduce_(0, lay + 1, torch.arange(m, dtype=torch.int64, device=lay.device), reduce="amin")
+    first = torch.where(counts > 0, first, torch.zeros_like(first))
+    return counts[1:].to(torch.int32), first[1:].to(torch.int32)
+
+
 def m_grouped_bf16_nt_contiguous(a: torch.Tensor, b: torch.Tensor, size_per_group: torch.Tensor, *,
                                  out: Optional[torch.Tensor] = None, grouped_layout: Optional[torch.Tensor] = None,
                                  block_m: int = 128, use_psum_layout: bool = False) -> torch.Tensor:
@@ -79,6 +95,11 @@ def m_grouped_bf16_nt_contiguous(a: torch.Tensor, b: torch.Tensor, size_per_grou
     _native.require_gpu(a, b, out)
     if not (a.is_contiguous() and b.is_contiguous() and out.is_contiguous()):
         raise ValueError("a, b and out must be contiguous")
+    if grouped_layout is not None and not use_psum_layout:  # per-row form: experts' regions in any order
+        rows, first = placement_from_layout(grouped_layout.to(a.device), g)
+        _native.call("tgg_m_grouped_gemm_placed", a.data_ptr(), b.data_ptr(), out.data_ptr(), rows.data_ptr(), 0,
+                     first.data_ptr(), g, m, n, k, _native.BF16, -1, _native.stream_of(a))
+        return out
     placed = size_per_group if grouped_layout is None else sizes_from_layout(grouped_layout, g, block_m, use_psum_layout)
     sizes, is64 = _sizes_on_device(placed, a.device)
     _native.call("tgg_m_grouped_gemm_padded", a.data_ptr(), b.data_ptr(), out.data_ptr(), sizes.data_ptr(), is64, g,
@@ -126,6 +147,12 @@ def m_grouped_fp8_nt_contiguous(a: Tuple[torch.Tensor, torch.Tensor], b: Tuple[t
     if sa.stride() != (1, m) and kb > 1:
         sa = sa.t().contiguous().t()
     sb = b_scale.to(torch.float32).contiguous()
+    if grouped_layout is not None and not use_psum_layout:  # per-row form: experts' regions in any order
+        rows, first = placement_from_layout(grouped_layout.to(a_codes.device), g)
+        _native.call("tgg_m_grouped_gemm_fp8_block_placed", a_codes.data_ptr(), sa.data_ptr(), b_codes.data_ptr(),
+                     sb.data_ptr(), out.data_ptr(), rows.data_ptr(), 0, first.data_ptr(), g, m, n, k, 1, -1,
+                     _native.stream_of(a_codes))
+        return out
     placed = size_per_group if grouped_layout is None else sizes_from_layout(grouped_layout, g, block_m, use_psum_layout)
     sizes, is64 = _sizes_on_device(placed, a_codes.device)
     _native.call("tgg_m_grouped_gemm_fp8_block", a_codes.data_ptr(), sa.data_ptr(), b_codes.data_ptr(),
