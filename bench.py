@@ -32,16 +32,16 @@ PEAK_HBM_GBS = 8000.0
 # plain 1 GiB device copy: x2.0 and x1.0).  The runs and their figures are listed in profiles/hbm_traffic.txt.
 # FETCH_SIZE includes L2 fills served by the memory-side cache, so these are upper bounds on DRAM traffic.
 MEASURED_TRAFFIC_GB = {
-    "bf16_m_grouped_gateup_nt": 11.71,
-    "bf16_m_grouped_gateup_nn": 11.55,
-    "bf16_m_grouped_gateup_fp8_out": 10.39,
-    "bf16_m_grouped_down_nt": 5.50,
-    "bf16_m_grouped_down_nn": 5.47,
-    "bf16_masked_decode": 2.59,
-    "bf16_k_grouped_wgrad": 34.00,
-    "fp8_block_m_grouped": 26.44,
-    "fp8_channel_m_grouped": 26.62,
-    "fp8_channel_k_grouped": 18.37,
+    "bf16_m_grouped_gateup_nt": 11.99,
+    "bf16_m_grouped_gateup_nn": 11.75,
+    "bf16_m_grouped_gateup_fp8_out": 10.61,
+    "bf16_m_grouped_down_nt": 5.42,
+    "bf16_m_grouped_down_nn": 5.36,
+    "bf16_masked_decode": 2.49,
+    "bf16_k_grouped_wgrad": 31.88,
+    "fp8_block_m_grouped": 28.91,
+    "fp8_channel_m_grouped": 27.94,
+    "fp8_channel_k_grouped": 18.23,
     "quant_trans128": 8.12,
     "moe_permute": 3.06,      # the row mover (the sort kernels move < 1 % of that)
     "moe_unpermute": 3.07,
