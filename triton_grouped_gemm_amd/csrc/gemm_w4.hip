@@ -17,11 +17,20 @@
 // waited for; copies every fourth multiply (the address unit takes 16 cycles per copy and its queue is short).
 // The slabs of all of a workgroup's tiles form one stream, as in gemm_fast.hip.
 //
+// The epilogue is deferred: a tile's results are converted, staged and stored between the multiplies of the next
+// tile's first K step (see "deferred epilogue" below), whose multiplies start from a zero addend instead of the
+// accumulators.  With one wave per SIMD an epilogue of its own leaves the matrix pipe idle for 12 us per tile
+// (headline 3.88 ms); deferred, conversion and staging disappear under the multiplies (what remains, 0.2 ms per
+// launch, is the issue of the stores themselves): headline 3.43 ms, K = 768 shape 2.78 -> 2.09 ms.  The eight-wave
+// kernel stands at 3.36 / 2.01 ms, so this kernel stays an opt-in path.
+//
 // What the compiler does not know about assembly statements, and how it is handled here:
 //   * a fragment read's result arrives later: every register a read targets passes through the wait statement
 //     ("+v") before a multiply may use it;
-//   * the multiplies write AGPRs: the last row block's accumulators pass through a statement of idle cycles before
-//     the epilogue (compiled code) reads them; accumulators are never the target of a load.
+//   * the multiplies write AGPRs: compiled code (the epilogue's conversions) reads a block's accumulators no sooner
+//     than 48 multiplies after the multiply that wrote them, except where a flush follows a tile directly: there the
+//     last row block's accumulators pass through a statement of idle cycles first.  Accumulators are never the
+//     target of a load.
 #include "fast_common.hpp"
 #include "launch.hpp"
 
@@ -35,6 +44,12 @@ constexpr int BK4 = 64;
 template <int DT> TGG_DEV void mfma_acc(f32x4_t& acc, const i32x4_t& w, const i32x4_t& x) {
   if (DT == DT_BF16) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(w), "v"(x));
   else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(w), "v"(x));
+}
+
+// The same with a zero addend: the first K step of a tile starts its accumulators afresh
+template <int DT> TGG_DEV void mfma_new(f32x4_t& acc, const i32x4_t& w, const i32x4_t& x) {
+  if (DT == DT_BF16) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(acc) : "v"(w), "v"(x));
+  else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(acc) : "v"(w), "v"(x));
 }
 
 // 16-byte fragment of a K-contiguous operand
@@ -218,15 +233,105 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   // Ends with the wait for those reads (and, when COPY is false, i.e. in front of the barrier, for this wave's copies
   // of the next slab): the registers the reads target pass through the wait statement, inside the same straight-line
   // code, before anything else may touch them.
-  auto kstep = [&](auto CURc, auto NKSc, auto MULc, auto COPYc, uint32_t nb_off, const SlabCopy& sc) {
+  // ---- deferred epilogue ---------------------------------------------------------------------------------------------
+  // A tile's results are stored during the first K step of the workgroup's next tile: with one wave per SIMD nothing
+  // else would keep the matrix pipe busy while a wave converts and stores its 128x128 block.  A lane owns row l16 and
+  // columns 16 j + 4 lg + (0..3) of each 16-row block i.  Strip i (one 16-row block, 128 columns) goes through the
+  // wave's LDS staging as two pieces of 64 columns and leaves as 16-byte stores covering 128-byte row segments.
+  // During the multiplies of row block i the blocks of strip i+1 are converted and staged one per multiply (their
+  // accumulators are the next to be overwritten: the first K step multiplies with a zero addend) and strip i,
+  // staged a row block earlier, is read back and stored.  The stores go through a buffer descriptor over the wave's
+  // block that ends with its last valid row; lanes whose columns lie beyond N get an out-of-range offset: no branches.
+  // Nothing pending = a descriptor of length zero.
+  i32x4_t pend_rs = make_rsrc32(0, 0);
+  int pend_cols = 0;
+  bool pending = false;
+  char* const stage = smem + C::EPI_OFF + wave * C::EPI_WAVE_BYTES;
+  // per-lane staging addresses and output offset, recomputed where a first K step or a flush begins
+  struct EpiLane { char* wr; const char* rd; int off; int ch8; };
+  auto epi_lane = [&]() {
+    int el = lane;
+    asm volatile("" : "+v"(el));
+    EpiLane e;
+    e.wr = stage + (el & 15) * C::EPI_PITCH + (el >> 4) * 8;
+    e.rd = stage + (el >> 3) * C::EPI_PITCH + (el & 7) * 16;
+    e.off = ((el >> 3) * p.N + (el & 7) * 8) * 2;
+    e.ch8 = (el & 7) * 8;
+    return e;
+  };
+  // block (i, j) -> staging piece j / 4; not before this point in the instruction stream
+  auto epi_cvt = [&](const EpiLane& e, int i, int j) {
+    asm volatile("" : "+a"(acc[i][j]));
+    *(uint2*)(e.wr + (j >> 2) * C::EPI_PIECE + (j & 3) * 32) = pack4<DT>(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+    asm volatile("" ::: "memory");
+  };
+  auto epi_read = [&](const EpiLane& e, int h, i32x4_t (&v)[2]) {
+#pragma unroll
+    for (int it = 0; it < 2; ++it) v[it] = *(const i32x4_t*)(e.rd + h * C::EPI_PIECE + it * 8 * C::EPI_PITCH);
+    asm volatile("" ::: "memory");
+  };
+  auto epi_store = [&](const EpiLane& e, int i, int h, int it, const i32x4_t& v) {
+    const int off = (64 * h + e.ch8 < pend_cols) ? e.off + ((16 * i + 8 * it) * p.N + 64 * h) * 2 : kNoFetch;
+    i32x4_t rs;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) rs[q] = __builtin_amdgcn_readfirstlane(pend_rs[q]);
+    // the wait states in front cover a descriptor written by a vector instruction just before (the compiler does not
+    // space what sits inside this statement), those behind it keep the data registers intact until the store has them
+    asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, 0 offen nt\n\ts_nop 1" : : "v"(v), "v"(off), "s"(rs) : "memory");
+  };
+  // everything that is pending, without multiplies to hide it under
+  auto epi_flush = [&]() {
+    if (pending) {
+      // the last row block's multiplies may have just been issued: give them time before compiled code reads the registers
+      asm volatile("s_nop 15\n\ts_nop 7" : "+a"(acc[7][0]), "+a"(acc[7][1]), "+a"(acc[7][2]), "+a"(acc[7][3]),
+                   "+a"(acc[7][4]), "+a"(acc[7][5]), "+a"(acc[7][6]), "+a"(acc[7][7]));
+      const EpiLane e = epi_lane();
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) epi_cvt(e, i, j);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          i32x4_t v[2];
+          epi_read(e, h, v);
+          epi_store(e, i, h, 0, v[0]);
+          epi_store(e, i, h, 1, v[1]);
+        }
+      }
+    }
+    pending = false;
+    pend_rs[2] = 0;
+  };
+
+  // EPI: the first K step of a tile -- multiplies start from zero, and the pending epilogue runs between them.
+  auto kstep = [&](auto CURc, auto NKSc, auto MULc, auto COPYc, uint32_t nb_off, const SlabCopy& sc, auto EPIc) {
     constexpr int CUR = decltype(CURc)::value, NKS = decltype(NKSc)::value;
-    constexpr bool MUL = decltype(MULc)::value, COPY = decltype(COPYc)::value;
+    constexpr bool MUL = decltype(MULc)::value, COPY = decltype(COPYc)::value, EPI = decltype(EPIc)::value;
+    static_assert(!EPI || MUL, "the deferred epilogue rides on a multiplying K step");
+    EpiLane e = {nullptr, nullptr, 0, 0};
+    i32x4_t v0[2], v1[2];
+    if (EPI) {
+      e = epi_lane();
+#pragma unroll
+      for (int j = 0; j < 8; ++j) epi_cvt(e, 0, j);  // strip 0 has no multiplies in front of it to hide under
+    }
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj) {
         const int j = (i & 1) ? 7 - jj : jj;  // snake order: one operand register changes per multiply
-        if (MUL) mfma_acc<DT>(acc[i][j], fb[CUR][j], fa[CUR][i]);
+        if (EPI) {
+          if (jj == 0) epi_read(e, 0, v0);            // strip i, staged during the previous row block
+          if (jj == 1) epi_read(e, 1, v1);
+          if (i < 7) epi_cvt(e, i + 1, jj);           // its piece's read-back has been issued (jj = 0: piece 0, jj = 4: piece 1)
+          if (jj == 3) epi_store(e, i, 0, 0, v0[0]);
+          if (jj == 4) epi_store(e, i, 0, 1, v0[1]);
+          if (jj == 5) epi_store(e, i, 1, 0, v1[0]);
+          if (jj == 6) epi_store(e, i, 1, 1, v1[1]);
+          mfma_new<DT>(acc[i][j], fb[CUR][j], fa[CUR][i]);
+        } else if (MUL) {
+          mfma_acc<DT>(acc[i][j], fb[CUR][j], fa[CUR][i]);
+        }
         const int n = i * 8 + jj;
 #define TGG_W4_RD(q) if (n + 1 == 3 * (q + 1)) read_frag(std::integral_constant<int, NKS>(), std::integral_constant<int, q>(), fa[CUR ^ 1], fb[CUR ^ 1], nb_off);
         TGG_W4_RD(0) TGG_W4_RD(1) TGG_W4_RD(2) TGG_W4_RD(3) TGG_W4_RD(4) TGG_W4_RD(5) TGG_W4_RD(6) TGG_W4_RD(7)
@@ -261,7 +366,7 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   }
   {
     SlabCopy none;
-    kstep(I1(), I0(), No(), No(), 0u, none);  // reads K step 0 of buffer 0 into set 0, multiplies nothing, waits for everything
+    kstep(I1(), I0(), No(), No(), 0u, none, No());  // reads K step 0 of buffer 0 into set 0, multiplies nothing, waits for everything
   }
   int ring = 0;
 
@@ -269,55 +374,30 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
     const Tile cur = tile_id == seen_id ? seen : sched_tile<C::BM, C::BN>(p, sched, tile_id);
     // a wave whose block of the tile has no rows or no columns multiplies nothing and stores nothing
     const bool active = wm0 < cur.rows && cur.n0 + wn0 < p.N;
-    for (int kt = 0; kt < kt_all; ++kt) {
+    if (!active) epi_flush();  // no multiplies in this tile to hide the pending stores under
+    // one slab; FIRST: the tile's first, whose first K step starts the accumulators afresh and carries the epilogue
+    auto slab = [&](auto FIRST) {
       const uint32_t cur_off = (ring & 1) * C::STAGE_BYTES, nxt_off = C::STAGE_BYTES - cur_off;
       const SlabCopy sc = begin_slab(ring & 1);  // descriptors of the slab after the next one, into the current slab's buffer
-      if (active) kstep(I0(), I1(), Yes(), No(), cur_off, sc);
-      else kstep(I0(), I1(), No(), No(), cur_off, sc);
+      if (active) kstep(I0(), I1(), Yes(), No(), cur_off, sc, FIRST);
+      else kstep(I0(), I1(), No(), No(), cur_off, sc, No());
       // set 1 is complete, this wave has read all it needs of the current slab, its copies of the next slab have landed
       asm volatile("s_barrier" ::: "memory");
-      if (active) kstep(I1(), I0(), Yes(), Yes(), nxt_off, sc);
-      else kstep(I1(), I0(), No(), Yes(), nxt_off, sc);
+      if (active) kstep(I1(), I0(), Yes(), Yes(), nxt_off, sc, No());
+      else kstep(I1(), I0(), No(), Yes(), nxt_off, sc, No());
       ++ring;
-    }
+    };
+    slab(Yes());
+    for (int kt = 1; kt < kt_all; ++kt) slab(No());
     if (!active) continue;
-
-    // ---- epilogue ------------------------------------------------------------------------------------------------
-    // the last row block's multiplies have just been issued: give them time before compiled code reads the registers
-    asm volatile("s_nop 15\n\ts_nop 7" : "+a"(acc[7][0]), "+a"(acc[7][1]), "+a"(acc[7][2]), "+a"(acc[7][3]),
-                 "+a"(acc[7][4]), "+a"(acc[7][5]), "+a"(acc[7][6]), "+a"(acc[7][7]));
-    // A lane owns row l16 and columns 16 j + 4 lg + (0..3) of each 16-row block i.  Pieces of 16 rows x 64 columns
-    // go through the wave's LDS staging (two pieces alternate) and leave as 16-byte stores covering 128-byte row segments.
-    int el = lane;
-    asm volatile("" : "+v"(el));
-    const int e16 = el & 15, eg = el >> 4;
-    char* const stage = smem + C::EPI_OFF + wave * C::EPI_WAVE_BYTES;
-    char* const c_tile = (char*)p.C + ((cur.row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2;
-    const bool full = cur.rows >= C::BM && cur.n0 + C::BN <= p.N;
-    const int st_r = el >> 3, st_ch = el & 7;  // a wave-wide read covers 8 rows of 8 chunks
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        char* const piece = stage + ((2 * i + h) & 1) * C::EPI_PIECE;
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          const int j = 4 * h + jj;
-          *(uint2*)(piece + e16 * C::EPI_PITCH + (16 * jj + 4 * eg) * 2) =
-              pack4<DT>(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
-          acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-        }
-#pragma unroll
-        for (int it = 0; it < 2; ++it) {
-          const int r = it * 8 + st_r;
-          const i32x4_t v = *(const i32x4_t*)(piece + r * C::EPI_PITCH + st_ch * 16);
-          const int row = wm0 + 16 * i + r, col = wn0 + 64 * h + st_ch * 8;
-          if (full || (row < cur.rows && cur.n0 + col < p.N))
-            store_c((i32x4_t*)(c_tile + ((int64_t)(16 * i + r) * p.N + 64 * h + st_ch * 8) * 2), v, p.store_nt);
-        }
-      }
-    asm volatile("s_nop 1" ::: "memory");  // cleared accumulators are read by the next tile's first multiplies
+    // what the next tile's first K step (or a flush) will store
+    const int rows_left = cur.rows - wm0;
+    pend_rs = make_rsrc32((uint64_t)p.C + (uint64_t)(((cur.row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2),
+                          (rows_left < 128 ? rows_left : 128) * p.N * 2);
+    pend_cols = __builtin_amdgcn_readfirstlane(p.N - cur.n0 - wn0);
+    pending = true;
   }
+  epi_flush();
   wait_vmcnt<0>();  // trailing zero-length copies still write LDS
 }
 
