@@ -28,11 +28,15 @@ def _codes_to_torch(codes: np.ndarray, fmt: str) -> torch.Tensor:
     return torch.from_numpy(codes.copy()).view(TORCH_FP8[fmt])
 
 
-@pytest.fixture(params=[0, 1], ids=["tuned", "generic"])
+@pytest.fixture(params=[0, 1, 2], ids=["tuned", "generic", "stream"])
 def variant(request, dev):
-    _native.set_option("force_generic", request.param)
+    """tuned: what a call gets by default; generic: the shape-agnostic kernel; stream: the weight-streaming
+    configuration (128-row tiles, three B slab buffers) forced onto every M-grouped launch, whatever the group sizes."""
+    _native.set_option("force_generic", int(request.param == 1))
+    _native.set_option("variant", 4 if request.param == 2 else 0)
     yield request.param
     _native.set_option("force_generic", 0)
+    _native.set_option("variant", 0)
 
 
 @pytest.mark.parametrize("fmt_a,fmt_b", [("e4m3fn", "e4m3fn"), ("e5m2", "e4m3fn"), ("e4m3fn", "e5m2"), ("e5m2", "e5m2")])

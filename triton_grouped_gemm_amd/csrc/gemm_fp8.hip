@@ -30,9 +30,12 @@ TGG_DEV void copy_b32_to_lds(i32x4_t rsrc, uint32_t lds_addr, int voff) {
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
 }
 
-template <int BM_, int BN_, int WM_, int WN_>
+// BST: slab buffers of the B operand.  2: the A slab, the B slab and the activation scales of a stage sit together, two
+// stages.  3 (the weight-streaming configuration, see gemm_fast.hip): A slabs and scales keep two buffers, the B
+// slabs get a ring of three of their own and their copies run a slab further ahead.
+template <int BM_, int BN_, int WM_, int WN_, int BST_ = 2>
 struct Fp8Cfg {
-  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BST = BST_;
   static constexpr int NWAVES = WM * WN;
   static constexpr int THREADS = NWAVES * 64;
   static constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128;
@@ -42,7 +45,11 @@ struct Fp8Cfg {
   static constexpr int TM = BM / WM / 16, TN = BN / WN / 16;  // 16x16 blocks per wave
   static constexpr int EPI_PITCH = TN * 32 + 16;  // staged strip of 16 rows x (16 TN) 16-bit outputs: row pitch in bytes
   static constexpr int EPI_WAVE_BYTES = 16 * EPI_PITCH;
-  static constexpr int SCHED_OFF = 2 * STAGE_BYTES;
+  static constexpr int SCHED_OFF = 2 * (A_BYTES + SA_BYTES) + BST * B_BYTES;
+  // byte offsets of A buffer a (0, 1), its scales, and B buffer b (0 .. BST-1)
+  static constexpr int a_off(int a) { return BST == 2 ? a * STAGE_BYTES : a * A_BYTES; }
+  static constexpr int s_off(int a) { return BST == 2 ? a * STAGE_BYTES + A_BYTES + B_BYTES : 2 * A_BYTES + a * SA_BYTES; }
+  static constexpr int b_off(int b) { return BST == 2 ? b * STAGE_BYTES + A_BYTES : 2 * (A_BYTES + SA_BYTES) + b * B_BYTES; }
   static constexpr int EPI_OFF = SCHED_OFF + (((int)sizeof(SchedTableT<kFastMaxGroups>) + 255) & ~255);
   static constexpr int SMEM_BYTES = EPI_OFF + NWAVES * EPI_WAVE_BYTES;
   static_assert(NI_A % NWAVES == 0 && NI_B % NWAVES == 0, "copies must divide evenly over waves");
@@ -50,7 +57,14 @@ struct Fp8Cfg {
   static_assert((BN / WN) <= 128, "a wave's columns must share one 128-wide weight scale block");
   static_assert(TM >= 4 && TM % 2 == 0 && TN >= 2, "the block schedule below alternates two A fragments");
   static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
+  static_assert(BST == 2 || BST == 3, "B slab buffers");
 };
+
+// s_waitcnt vmcnt(N) lgkmcnt(0): all LDS reads and all but the N most recent vector-memory operations are complete
+template <int N> TGG_DEV void wait_vmcnt_lgkmcnt0() {
+  static_assert(N >= 0 && N < 64, "vmcnt range");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4));
+}
 
 // FA / FB: 0 = e4m3fn, 1 = e5m2 (the cbsz / blgp format codes of the f8f6f4 MFMA).
 // The whole kernel but for the group table, which the caller has built at byte SCHED_AT of the workgroup's LDS.
@@ -61,6 +75,8 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   typedef Operand<C::BM, true> OpA;
   typedef Operand<C::BN, true> OpB;
   constexpr bool BLOCK = EPI == EPI_BLOCK;
+  constexpr bool DEEP = C::BST == 3;  // three B slab buffers, B copies a slab further ahead (see gemm_fast.hip)
+  static_assert(!DEEP || !KGROUP, "the weight-streaming configuration is M-grouped");
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const auto& sched = *reinterpret_cast<const SchedTableT<kFastMaxGroups>*>(smem + SCHED_AT);
@@ -132,8 +148,17 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   // This is an ordinary vector load, so the compiler waits for *all* outstanding vector memory
   // traffic at its first use; it is therefore fetched one tile ahead and first touched right after
   // a point where this wave has waited for everything anyway.
+  // With the deep ring a wave never waits for *everything* (its newest B copies stay in flight), so there the
+  // load is inline assembly as well: loads complete in order, and the value is first used a tile later, behind
+  // several of the stream's own waits.
   auto load_sbv = [&](const Tile& t) {
     const int64_t idx = ((int64_t)t.g * nblocks + ((t.n0 + wn0) >> 7)) * kblocks;
+    if (DEEP && BLOCK) {
+      float v;
+      const float* src = p.sb + idx + (lane < kblocks ? lane : 0);
+      asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(src) : "memory");
+      return v;
+    }
     return (BLOCK && lane < kblocks) ? p.sb[idx + lane] : 0.f;
   };
 
@@ -148,6 +173,25 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   // reaches that tile later and reuses the lookup instead of repeating its chain of dependent LDS reads.
   Tile nt;
   int nt_id = -1;
+  // DEEP: the B copies have a cursor of their own, one slab ahead of `feed` (which then serves A and the scales)
+  TileIo feedb;
+  int feedb_id = -1;
+  auto feedb_seek = [&](int id) {
+    feedb.kt_n = 0;
+    feedb.issued = 0;
+    feedb.a_base = feedb.b_base = feedb.s_base = (uint64_t)p.A;
+    feedb.a_left = feedb.b_left = 0;
+    feedb.s_bytes = 0;
+    feedb.k_left = 0;
+    for (; id < walk.end; id += walk.stride) {
+      const Tile tt = id == nt_id ? nt : sched_tile<C::BM, C::BN>(p, sched, id);
+      if (slabs_of(tt) > 0) {
+        feedb = make_io(tt);
+        break;
+      }
+    }
+    feedb_id = id;
+  };
   auto feed_seek = [&](int id) {
     feed.kt_n = 0;
     feed.issued = 0;
@@ -166,19 +210,34 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   };
   struct SlabCopy {
     i32x4_t ra, rb, rs;
-    uint32_t base;
-    bool tail;  // the tile's last slab, cut short by K
+    uint32_t base, base_s, base_b;  // LDS addresses of the A slab, its scales and the B slab
+    bool tail, tail_b;  // the tile's last slab, cut short by K (DEEP: A and B are slabs of different numbers)
     int chunks; // K-grouped: 16-byte chunks of this slab that belong to the group (8 but for a group's last slab)
   };
   constexpr int CA = C::NI_A / C::NWAVES, CB = C::NI_B / C::NWAVES, CS = BLOCK ? 1 : 0, NC = CS + CA + CB;
-  auto begin_slab = [&](int buf) {
+  auto begin_b = [&](SlabCopy& sc, int buf_b) {  // DEEP: the next B slab of the B cursor, into B buffer buf_b
+    const bool live = feedb.issued < feedb.kt_n;
+    sc.rb = make_rsrc32(feedb.b_base, live ? feedb.b_left : 0);
+    sc.base_b = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_addr + C::b_off(buf_b)));  // wave-uniform: goes into m0
+    sc.tail_b = tail_chunks != 0 && feedb.issued + 1 == feedb.kt_n;
+    feedb.b_base += BKB;
+    feedb.b_left -= BKB;
+    feedb.issued += 1;
+    if (live && feedb.issued >= feedb.kt_n) feedb_seek(feedb_id + walk.stride);
+  };
+  auto begin_slab = [&](int buf, int buf_b = 0) {
     SlabCopy sc;
     const bool live = feed.issued < feed.kt_n;
     sc.ra = make_rsrc32(feed.a_base, live ? feed.a_left : 0);
-    sc.rb = make_rsrc32(feed.b_base, live ? feed.b_left : 0);
     sc.rs = make_rsrc32(feed.s_base, live ? feed.s_bytes : 0);
-    sc.base = smem_addr + buf * C::STAGE_BYTES;
+    sc.base = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_addr + C::a_off(buf)));
+    sc.base_s = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_addr + C::s_off(buf)));
     sc.tail = tail_chunks != 0 && feed.issued + 1 == feed.kt_n;
+    if (!DEEP) {
+      sc.rb = make_rsrc32(feed.b_base, live ? feed.b_left : 0);
+      sc.base_b = (uint32_t)__builtin_amdgcn_readfirstlane((int)(smem_addr + C::b_off(buf)));
+      sc.tail_b = sc.tail;
+    }
     sc.chunks = KGROUP ? (feed.k_left >= BKB ? 8 : (feed.k_left > 0 ? feed.k_left >> 4 : 0)) : 8;
     feed.k_left -= BKB;
     feed.a_base += BKB;
@@ -188,6 +247,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
     feed.s_base += (uint64_t)p.m_total * 4;
     feed.issued += 1;
     if (live && feed.issued >= feed.kt_n) feed_seek(feed_id + walk.stride);
+    if (DEEP) begin_b(sc, buf_b);
     return sc;
   };
   auto copy_k = [&](const SlabCopy& sc, int k) {
@@ -195,7 +255,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
       // activation scales of the slab's rows: wave w fetches rows 64 w .. 64 w + 63; spare waves issue an
       // out-of-range copy into a sink so that every wave has the same number of copies in flight
       const bool mine = wave * 64 < C::BM;
-      copy_b32_to_lds(sc.rs, sc.base + C::A_BYTES + C::B_BYTES + (mine ? wave * 256 : C::BM * 4),
+      copy_b32_to_lds(sc.rs, sc.base_s + (mine ? wave * 256 : C::BM * 4),
                       mine ? (wave * 64 + lane) * 4 : kNoFetch);
     } else if (k < CS + CA) {
       const int idx = wave + (k - CS) * C::NWAVES;  // wave-uniform
@@ -203,8 +263,8 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
       copy_b128_to_lds(sc.ra, sc.base + idx * 1024, v0 + idx * OpA::RPI * (int)ld);
     } else {
       const int idx = wave + (k - CS - CA) * C::NWAVES;
-      const int v0 = KGROUP ? (b_chunk >= sc.chunks ? kNoFetch : b_voff) : (sc.tail ? b_voff_tail : b_voff);
-      copy_b128_to_lds(sc.rb, sc.base + C::A_BYTES + idx * 1024, v0 + idx * OpB::RPI * (int)ld);
+      const int v0 = KGROUP ? (b_chunk >= sc.chunks ? kNoFetch : b_voff) : (sc.tail_b ? b_voff_tail : b_voff);
+      copy_b128_to_lds(sc.rb, sc.base_b + idx * 1024, v0 + idx * OpB::RPI * (int)ld);
     }
   };
 
@@ -218,15 +278,24 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   // multiply 4 % slower: the address unit's queue is short, see gemm_fast.hip).
   // Block scaling: every multiply starts from zero and its result is folded into the accumulators, scaled, two
   // multiplies later.
+  // DEEP: per slab the scale, A and then B copies go out, the B copies for a slab one further ahead; the wait lets
+  // the CB most recent copies -- those B copies -- stay in flight (loads complete in order).
+  constexpr int WAIT_N = DEEP ? CB : 0;
+  if (DEEP) feedb_seek(walk.first);
   feed_seek(walk.first);
   {
-    const SlabCopy s0 = begin_slab(0);
+    SlabCopy s0 = begin_slab(0, 0);
 #pragma unroll
     for (int k = 0; k < NC; ++k) copy_k(s0, k);
+    if (DEEP) {  // B slab 1 as well: from here on the B cursor is a slab ahead
+      begin_b(s0, 1);
+#pragma unroll
+      for (int k = CS + CA; k < NC; ++k) copy_k(s0, k);
+    }
   }
   wait_vmcnt<0>();
   __syncthreads();
-  SlabCopy sc = begin_slab(1);
+  SlabCopy sc = begin_slab(1, 2);
   // copy k of `sc`, if there is one (k is a compile-time constant at every call site)
   auto copy_at = [&](int k) {
     if (k < NC) {
@@ -239,14 +308,16 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   for (int k = 0; k < C::TN; ++k) copy_at(k);
   i32x8_t fb[C::TN], fa[2];
 #pragma unroll
-  for (int j = 0; j < C::TN; ++j) fb[j] = load_frag(smem + C::A_BYTES + (wn0 + 16 * j) * 128);
-  fa[0] = load_frag(smem + wm0 * 128);
+  for (int j = 0; j < C::TN; ++j) fb[j] = load_frag(smem + C::b_off(0) + (wn0 + 16 * j) * 128);
+  fa[0] = load_frag(smem + C::a_off(0) + wm0 * 128);
   int ring = 0;
+  int ring3 = 0;  // ring % 3 (DEEP: the B buffer of the current slab)
 
   float sbv_next = 0.f;
   if (walk.first < walk.end) {
     nt = sched_tile<C::BM, C::BN>(p, sched, walk.first);
     sbv_next = load_sbv(nt);
+    if (DEEP && BLOCK) wait_vmcnt<0>();  // there the load is not the compiler's to wait for, and the first slab reads it
   }
   // The accumulators start at zero and the epilogue clears every strip right after it has converted it.
   f32x4_t acc[C::TM][C::TN];
@@ -283,8 +354,8 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
           copy_at(k);
           __builtin_amdgcn_s_sleep(1);  // paced: the address unit's queue is shared with the working waves
         }
-        const SlabCopy scn = begin_slab(ring & 1);
-        wait_vmcnt<0>();
+        const SlabCopy scn = begin_slab(ring & 1, ring3);
+        wait_vmcnt<WAIT_N>();
         if (BLOCK) asm volatile("" : "+v"(sbv_next));
         __syncthreads();
         sc = scn;
@@ -294,12 +365,12 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
           __builtin_amdgcn_s_sleep(1);
         }
         ++ring;
+        ring3 = ring3 == 2 ? 0 : ring3 + 1;
       }
       if (kt_n > 0) {
-        const char* sn = smem + (ring & 1) * C::STAGE_BYTES;
 #pragma unroll
-        for (int j = 0; j < C::TN; ++j) fb[j] = load_frag(sn + C::A_BYTES + (wn0 + 16 * j) * 128);
-        fa[0] = load_frag(sn + wm0 * 128);
+        for (int j = 0; j < C::TN; ++j) fb[j] = load_frag(smem + C::b_off(DEEP ? ring3 : (ring & 1)) + (wn0 + 16 * j) * 128);
+        fa[0] = load_frag(smem + C::a_off(ring & 1) + wm0 * 128);
       }
       continue;
     }
@@ -309,15 +380,17 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
     f32x4_t part[4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
     float s_carry = 0.f;
     for (int kt = 0; kt < kt_n; ++kt) {
-      const char* sa = smem + (ring & 1) * C::STAGE_BYTES;
-      const char* sn = smem + ((ring + 1) & 1) * C::STAGE_BYTES;
+      const int ring3n = ring3 == 2 ? 0 : ring3 + 1;
+      const char* sa = smem + C::a_off(ring & 1);                            // A slab of the current slab
+      const char* sn = smem + C::a_off((ring + 1) & 1);                      // ... and of the next
+      const char* sbn = smem + C::b_off(DEEP ? ring3n : ((ring + 1) & 1));   // B slab of the next slab
       // row scales of the slab: read here, multiplied with the weight scale only after the row block's first
       // multiply has been issued, so that the wait for the reads does not sit in front of the slab's first multiply
       float srow[C::TM];
       float sb_cur = 0.f;
       if (BLOCK) {
         sb_cur = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sbv), kt));
-        const float* ss = (const float*)(sa + C::A_BYTES + C::B_BYTES) + wm0 + l16;
+        const float* ss = (const float*)(smem + C::s_off(ring & 1)) + wm0 + l16;
 #pragma unroll
         for (int i = 0; i < C::TM; ++i) srow[i] = ss[16 * i];
       }
@@ -330,8 +403,8 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
         } else {
           // this wave's share of the next slab has landed, and its reads of the current slab (the last A
           // fragment was requested a row block ago) are complete: after the barrier the buffer is overwritten
-          wait_vmcnt0_lgkmcnt0();
-          if (BLOCK) asm volatile("" : "+v"(sbv_next));  // nothing of this wave is in flight: touching it costs no wait
+          wait_vmcnt_lgkmcnt0<WAIT_N>();
+          if (BLOCK) asm volatile("" : "+v"(sbv_next));  // everything older than the newest B copies has landed: touching it costs no wait
           __syncthreads();
           sc = scn;
           fa[0] = load_frag(sn + wm0 * 128);
@@ -352,9 +425,9 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
           __builtin_amdgcn_sched_barrier(0);
           if (i == C::TM - 1) {
             copy_at(jj);
-            fb[j] = load_frag(sn + C::A_BYTES + (wn0 + 16 * j) * 128);
+            fb[j] = load_frag(sbn + (wn0 + 16 * j) * 128);
           } else {
-            if (n == C::TN * (C::TM - 2) + 1) scn = begin_slab(ring & 1);  // scalar work under a multiply
+            if (n == C::TN * (C::TM - 2) + 1) scn = begin_slab(ring & 1, ring3);  // scalar work under a multiply
             // block-scaled: one copy per multiply; per-channel (no folds between the multiplies, so the copies of
             // all waves come closer together and crowd the address unit's queue): one per two multiplies, +0.9 %
             if (BLOCK) copy_at(C::TN + n);
@@ -383,6 +456,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
       }
       if (BLOCK) s_carry = srow[C::TM - 1];
       ++ring;
+      ring3 = ring3n;
     }
     if (BLOCK) {
 #pragma unroll
@@ -467,26 +541,35 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
 // gemm_fast.hip): narrow tiles when all of them fit one round of the persistent workgroups; otherwise wide tiles,
 // with the sit-out path when at least one tile in eight is at most half full (groups whose size modulo 256 lies
 // in 1..128: decode-sized groups), without it otherwise.
-template <class CW, class CN, int FA, int FB, int EPI, int OUT>
+// A fourth body, the weight-streaming configuration CS (128-row tiles, three B slab buffers, see gemm_fast.hip), runs
+// when no group has more than 128 rows and the narrow tiles do not fit one round: every group then has at most one
+// row tile of either height, so the same group table serves it.
+template <class CW, class CN, class CS, int FA, int FB, int EPI, int OUT>
 __global__ __launch_bounds__(CW::THREADS) void gemm_fp8_auto_kernel(const GemmParams p) {
   static_assert(CW::BM == CN::BM && CW::THREADS == CN::THREADS, "one group table, one launch shape");
   static_assert(CN::SMEM_BYTES <= CW::SCHED_OFF, "the narrow configuration must not reach the shared group table");
+  static_assert(CS::THREADS == CW::THREADS && CS::SCHED_OFF <= CW::SCHED_OFF && CS::SMEM_BYTES <= CW::SMEM_BYTES,
+                "the weight-streaming configuration shares the launch shape and must not reach the group table");
   static_assert(CW::THREADS >= kFastMaxGroups && CW::BM == 256, "one group per thread in the count below");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + CW::SCHED_OFF);
   sched_init<CW::BM>(p, sched);
-  int half_full = 0;
+  int half_full = 0, big = 0;
   if ((int)threadIdx.x < p.G) {
     const int r = sched.rows[threadIdx.x] & 255;
     half_full = r >= 1 && r <= 128;
+    big = sched.rows[threadIdx.x] > CS::BM;
   }
   const int n_half_full = __syncthreads_count(half_full);
+  const bool stream = __syncthreads_or(big) == 0;
   const bool narrow = sched_num_tiles<CN::BM, CN::BN>(p, sched) <= (int64_t)gridDim.x;
   const bool sit_out = n_half_full * 8 >= sched.tile0[p.G];
   if (__builtin_expect(!narrow && !sit_out, 1))  // marked likely: the register allocator then favours this body's loops
     gemm_fp8_body<CW, FA, FB, EPI, OUT, false, CW::SCHED_OFF, false>(p);
   else if (narrow)
     gemm_fp8_body<CN, FA, FB, EPI, OUT, false, CW::SCHED_OFF, true>(p);
+  else if (stream)
+    gemm_fp8_body<CS, FA, FB, EPI, OUT, false, CW::SCHED_OFF, true>(p);
   else
     gemm_fp8_body<CW, FA, FB, EPI, OUT, false, CW::SCHED_OFF, true>(p);
 }
@@ -509,17 +592,20 @@ int launch_fp8_kernel(Kern kern, int smem_bytes, int threads, bool (&attr_set)[6
 
 typedef Fp8Cfg<256, 256, 2, 4> Fp8Wide;
 typedef Fp8Cfg<256, 128, 2, 4> Fp8Narrow;
+typedef Fp8Cfg<128, 256, 2, 4, 3> Fp8Stream;
 
-int g_fp8_variant = 0;  // 0: chosen on the device (M-grouped), 1: narrow, 2: wide
+int g_fp8_variant = 0;  // 0: chosen on the device (M-grouped), 1: narrow, 2: wide, 4: weight-streaming configuration
 
 // M-grouped launches choose the tile width on the device; K-grouped ones (tile count known to the host, tile cost
 // set by the group's token count) use the wide tiles.
 template <int FA, int FB, int EPI, int OUT, bool KGROUP>
 int launch_fp8_cfg(const GemmParams& p, hipStream_t s) {
-  static bool attr_auto[64] = {false}, attr_wide[64] = {false}, attr_narrow[64] = {false};
+  static bool attr_auto[64] = {false}, attr_wide[64] = {false}, attr_narrow[64] = {false}, attr_stream[64] = {false};
   if constexpr (!KGROUP) {
     if (g_fp8_variant == 0)
-      return launch_fp8_kernel(gemm_fp8_auto_kernel<Fp8Wide, Fp8Narrow, FA, FB, EPI, OUT>, Fp8Wide::SMEM_BYTES, Fp8Wide::THREADS, attr_auto, p, s);
+      return launch_fp8_kernel(gemm_fp8_auto_kernel<Fp8Wide, Fp8Narrow, Fp8Stream, FA, FB, EPI, OUT>, Fp8Wide::SMEM_BYTES, Fp8Wide::THREADS, attr_auto, p, s);
+    if (g_fp8_variant == 4)
+      return launch_fp8_kernel(gemm_fp8_kernel<Fp8Stream, FA, FB, EPI, OUT, false>, Fp8Stream::SMEM_BYTES, Fp8Stream::THREADS, attr_stream, p, s);
     if (g_fp8_variant == 1)
       return launch_fp8_kernel(gemm_fp8_kernel<Fp8Narrow, FA, FB, EPI, OUT, false>, Fp8Narrow::SMEM_BYTES, Fp8Narrow::THREADS, attr_narrow, p, s);
   }
