@@ -150,16 +150,16 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   // a point where this wave has waited for everything anyway.
   // With the deep ring a wave never waits for *everything* (its newest B copies stay in flight), so there the
   // load is inline assembly as well: loads complete in order, and the value is first used a tile later, behind
-  // several of the stream's own waits.
-  auto load_sbv = [&](const Tile& t) {
+  // several of the stream's own waits.  It loads into the variable's own register ("+v"): the compiler, which
+  // takes the statement's result for available at once, then has no reason to copy it anywhere before it has arrived.
+  auto load_sbv = [&](const Tile& t, float& dst) {
     const int64_t idx = ((int64_t)t.g * nblocks + ((t.n0 + wn0) >> 7)) * kblocks;
     if (DEEP && BLOCK) {
-      float v;
       const float* src = p.sb + idx + (lane < kblocks ? lane : 0);
-      asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(src) : "memory");
-      return v;
+      asm volatile("global_load_dword %0, %1, off" : "+v"(dst) : "v"(src) : "memory");
+    } else {
+      dst = (BLOCK && lane < kblocks) ? p.sb[idx + lane] : 0.f;
     }
-    return (BLOCK && lane < kblocks) ? p.sb[idx + lane] : 0.f;
   };
 
   // The copy stream (see gemm_fast.hip): slab q of the workgroup's whole slab sequence lives in buffer q % 2.
@@ -316,7 +316,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   float sbv_next = 0.f;
   if (walk.first < walk.end) {
     nt = sched_tile<C::BM, C::BN>(p, sched, walk.first);
-    sbv_next = load_sbv(nt);
+    load_sbv(nt, sbv_next);
     if (DEEP && BLOCK) wait_vmcnt<0>();  // there the load is not the compiler's to wait for, and the first slab reads it
   }
   // The accumulators start at zero and the epilogue clears every strip right after it has converted it.
@@ -341,7 +341,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
     if (tile_id + walk.stride < walk.end) {
       nt = sched_tile<C::BM, C::BN>(p, sched, tile_id + walk.stride);
       nt_id = tile_id + walk.stride;
-      sbv_next = load_sbv(nt);
+      load_sbv(nt, sbv_next);
     }
 
     // A wave whose block of the tile has no rows (groups of at most BM / WM rows) or no columns sits the tile
