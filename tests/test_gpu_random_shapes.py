@@ -23,6 +23,16 @@ def dev():
     return torch.device("cuda:0")
 
 
+def _half_ulp_of_fp32(out, ref32):
+    """Every element within half an output ulp (+2 %, + accumulation-order noise) of an fp32 product computed by a
+    library routine (torch's matmul on the GPU): independent of both kernels of this library."""
+    if out.numel() == 0:
+        return True
+    eps = 2.0 ** -8 if out.dtype == torch.bfloat16 else 2.0 ** -11
+    err = (out.float() - ref32).abs()
+    return bool((err <= ref32.abs() * eps * 1.02 + 2e-6 * ref32.abs().max()).all())
+
+
 def _both(fn):
     _native.set_option("force_generic", 1)
     try:
@@ -60,11 +70,23 @@ def test_tuned_equals_generic_on_random_shapes(dev, seed):
                 finally:
                     _native.set_option("four_wave", 0)
                 assert torch.equal(out4, ref), f"four-wave kernel differs: seed {seed} case {case} G={G} N={N} K={K} {dt}"
+            start = 0
+            for g, n_rows in enumerate(sizes):  # and against torch's fp32 product, group by group
+                if n_rows:
+                    w = b[g].float()
+                    assert _half_ulp_of_fp32(out[start:start + n_rows], a[start:start + n_rows].float() @ (w.t() if tb else w)), \
+                        f"seed {seed} case {case} group {g}"
+                start += n_rows
         elif kind == 1 and M > 0:
             Md = 8 * rng.randint(1, 80)
             a = torch.randn(M, Md, device=dev).to(dt)
             b = torch.randn(M, N, device=dev).to(dt)
             out, ref = _both(lambda: k_grouped_gemm(a, b, st))
+            start = 0
+            for g, n_rows in enumerate(sizes):
+                exact = a[start:start + n_rows].float().t() @ b[start:start + n_rows].float()
+                assert _half_ulp_of_fp32(out[g], exact), f"seed {seed} case {case} group {g}"
+                start += n_rows
         else:
             m_max = 128 * rng.randint(1, 4)
             mm = torch.tensor([rng.randint(0, m_max) for _ in range(G)], dtype=torch.int32, device=dev)
@@ -77,6 +99,10 @@ def test_tuned_equals_generic_on_random_shapes(dev, seed):
                 return o
 
             out, ref = _both(masked)
+            for g, cnt in enumerate(mm.tolist()):
+                rows = out[g * m_max:g * m_max + cnt]
+                assert _half_ulp_of_fp32(rows, a[g * m_max:g * m_max + cnt].float() @ b[g].float().t()), f"seed {seed} case {case} group {g}"
+                assert bool((out[g * m_max + cnt:(g + 1) * m_max] == 7.0).all())
         assert torch.equal(out, ref), f"seed {seed} case {case} kind {kind} G={G} N={N} K={K} {dt}"
 
 
@@ -98,7 +124,7 @@ def test_tile_configurations_agree(dev, G, per_group, N, K):
     finally:
         _native.set_option("force_generic", 0)
     try:
-        for v in (0, 1, 2):  # chosen on the device, always narrow, always wide
+        for v in (0, 1, 2, 4):  # chosen on the device, always narrow, always wide, always the weight-streaming configuration
             _native.set_option("variant", v)
             assert torch.equal(m_grouped_gemm(a, b, st, True), ref), v
             assert torch.equal(k_grouped_gemm(ak, bk, st), refk), v
