@@ -542,8 +542,8 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
 // with the sit-out path when at least one tile in eight is at most half full (groups whose size modulo 256 lies
 // in 1..128: decode-sized groups), without it otherwise.
 // A fourth body, the weight-streaming configuration CS (128-row tiles, three B slab buffers, see gemm_fast.hip), runs
-// when no group has more than 128 rows and the narrow tiles do not fit one round: every group then has at most one
-// row tile of either height, so the same group table serves it.
+// when the groups are decode-sized (the 128-row cut has at most a quarter more tiles than the 256-row cut) and the
+// narrow tiles do not fit one round; the table's tile prefix is rebuilt for its tile height when that differs.
 template <class CW, class CN, class CS, int FA, int FB, int EPI, int OUT>
 __global__ __launch_bounds__(CW::THREADS) void gemm_fp8_auto_kernel(const GemmParams p) {
   static_assert(CW::BM == CN::BM && CW::THREADS == CN::THREADS, "one group table, one launch shape");
@@ -554,22 +554,30 @@ __global__ __launch_bounds__(CW::THREADS) void gemm_fp8_auto_kernel(const GemmPa
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + CW::SCHED_OFF);
   sched_init<CW::BM>(p, sched);
-  int half_full = 0, big = 0;
+  int half_full = 0;
+  if (threadIdx.x == 0) sched.pad_ = 0;
+  __syncthreads();
   if ((int)threadIdx.x < p.G) {
-    const int r = sched.rows[threadIdx.x] & 255;
+    const int rows = sched.rows[threadIdx.x];
+    const int r = rows & 255;
     half_full = r >= 1 && r <= 128;
-    big = sched.rows[threadIdx.x] > CS::BM;
+    const int extra = (rows + CS::BM - 1) / CS::BM - (rows + CW::BM - 1) / CW::BM;
+    if (extra) atomicAdd(&sched.pad_, extra);  // tiles that the 128-row cut has over the 256-row cut
   }
   const int n_half_full = __syncthreads_count(half_full);
-  const bool stream = __syncthreads_or(big) == 0;
+  const bool stream = sched.pad_ * 4 <= sched.tile0[p.G];
   const bool narrow = sched_num_tiles<CN::BM, CN::BN>(p, sched) <= (int64_t)gridDim.x;
   const bool sit_out = n_half_full * 8 >= sched.tile0[p.G];
   if (__builtin_expect(!narrow && !sit_out, 1))  // marked likely: the register allocator then favours this body's loops
     gemm_fp8_body<CW, FA, FB, EPI, OUT, false, CW::SCHED_OFF, false>(p);
   else if (narrow)
     gemm_fp8_body<CN, FA, FB, EPI, OUT, false, CW::SCHED_OFF, true>(p);
-  else if (stream)
+  else if (stream) {
+    if (sched.pad_ != 0) {  // some group has more than one 128-row tile: the tile prefix for this tile height
+      sched_retile<CS::BM>(p, sched);
+    }
     gemm_fp8_body<CS, FA, FB, EPI, OUT, false, CW::SCHED_OFF, true>(p);
+  }
   else
     gemm_fp8_body<CW, FA, FB, EPI, OUT, false, CW::SCHED_OFF, true>(p);
 }
