@@ -645,14 +645,14 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fast_kernel(const GemmParams 
 // Several tile configurations in one kernel, chosen per launch from the group sizes, which only the device knows:
 //   * the narrow tiles (half the columns) when all of them fit into a single round of the persistent workgroups
 //     -- twice as many workgroups then have work, and a narrow tile costs about 0.7 of a wide one;
-//   * otherwise, when the groups are decode-sized (the launch streams weights), the weight-streaming configuration
+//   * otherwise, when the groups are small (the launch streams weights), the weight-streaming configuration
 //     CS -- 128-row tiles and a ring of three B slabs whose copies run a slab further ahead, i.e. twice the weight
-//     bytes in flight per CU: 5-15 % faster there (up to 6 TB/s of weights).  Decode-sized: cutting the groups into
-//     128-row tiles gives at most a quarter more tiles than cutting them into 256-row tiles, i.e. few groups have
-//     more than 128 rows (each of those re-reads its weights once more, which is what the 128-row tiles cost);
+//     bytes in flight per CU: 5-30 % faster there (up to 6 TB/s of weights).  A 128-row tile costs about 0.7 of a
+//     256-row one, so CS runs when its rounds of the persistent workgroups, times 0.7, are no more than the wide
+//     configuration's rounds (see sched_short_tiles_pay): groups of up to about 200 rows on average;
 //   * the wide tiles otherwise.
 // Wide and narrow use BM-row tiles, so one group table serves both; for CS the table's tile prefix is rebuilt for
-// its tile height when it differs (some group above 128 rows).  The table sits where the wide configuration keeps
+// its tile height when it differs (some group above 128 rows; sched_init has computed it alongside).  The table sits where the wide configuration keeps
 // it, past everything the others touch.  CS = void: no weight-streaming configuration (K-grouped).
 template <class CW, class CN, class CS, int DT, int LAYOUT>
 __global__ __launch_bounds__(CW::THREADS) void gemm_fast_auto_kernel(const GemmParams p) {
@@ -660,28 +660,19 @@ __global__ __launch_bounds__(CW::THREADS) void gemm_fast_auto_kernel(const GemmP
   static_assert(CN::SMEM_BYTES <= CW::SCHED_OFF, "the narrow configuration must not reach the shared group table");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + CW::SCHED_OFF);
-  sched_init<CW::BM>(p, sched);
+  const int32_t half_tile0 = sched_init<CW::BM>(p, sched);
   bool stream = false;
   if constexpr (!std::is_void<CS>::value) {
     static_assert(CS::THREADS == CW::THREADS && CS::SCHED_OFF == CW::SCHED_OFF && CS::SMEM_BYTES <= CW::SMEM_BYTES,
                   "the weight-streaming configuration shares the launch shape and the group table's place");
-    static_assert(CW::THREADS >= kFastMaxGroups, "one group per thread in the count below");
-    // tiles that the 128-row cut has over the 256-row cut, summed over the groups in the table's spare word
-    if (threadIdx.x == 0) sched.pad_ = 0;
-    __syncthreads();
-    if ((int)threadIdx.x < p.G) {
-      const int r = sched.rows[threadIdx.x];
-      const int extra = (r + CS::BM - 1) / CS::BM - (r + CW::BM - 1) / CW::BM;
-      if (extra) atomicAdd(&sched.pad_, extra);
-    }
-    __syncthreads();
-    stream = sched.pad_ * 4 <= sched.tile0[p.G];
+    static_assert(CW::THREADS >= kFastMaxGroups && CS::BM * 2 == CW::BM, "sched_init's half-height prefix is CS's");
+    stream = sched_short_tiles_pay<CW::BN>(p, sched);
   }
   if (__builtin_expect(sched_num_tiles<CN::BM, CN::BN>(p, sched) > (int64_t)gridDim.x, 1)) {
     if constexpr (!std::is_void<CS>::value) {
       if (__builtin_expect(stream, 0)) {
         if (sched.pad_ != 0) {  // some group has more than one 128-row tile: the tile prefix for this tile height
-          sched_retile<CS::BM>(p, sched);
+          sched_use_half_height(p, sched, half_tile0);
         }
         gemm_fast_body<CS, DT, LAYOUT, false, CW::SCHED_OFF>(p);
         return;

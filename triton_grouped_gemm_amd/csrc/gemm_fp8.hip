@@ -537,46 +537,42 @@ __global__ __launch_bounds__(C::THREADS) void gemm_fp8_kernel(const GemmParams p
   gemm_fp8_body<C, FA, FB, EPI, OUT, KGROUP, C::SCHED_OFF, false>(p);
 }
 
-// Three bodies in one kernel, chosen per launch on the device from the group sizes (see gemm_fast_auto_kernel in
+// Several bodies in one kernel, chosen per launch on the device from the group sizes (see gemm_fast_auto_kernel in
 // gemm_fast.hip): narrow tiles when all of them fit one round of the persistent workgroups; otherwise wide tiles,
-// with the sit-out path when at least one tile in eight is at most half full (groups whose size modulo 256 lies
-// in 1..128: decode-sized groups), without it otherwise.
+// with the sit-out path when at least one tile in eight is at most half full (groups whose size modulo the tile
+// height lies in the lower half: decode-sized groups), without it otherwise.
 // A fourth body, the weight-streaming configuration CS (128-row tiles, three B slab buffers, see gemm_fast.hip), runs
-// when the groups are decode-sized (the 128-row cut has at most a quarter more tiles than the 256-row cut) and the
-// narrow tiles do not fit one round; the table's tile prefix is rebuilt for its tile height when that differs.
+// when the narrow tiles do not fit one round and its rounds, at 0.7 of a wide tile's cost each, are no more than the
+// wide configuration's (sched_short_tiles_pay), without the sit-out path (measured: no gain there); the table's tile
+// prefix is switched to its tile height when that differs.
 template <class CW, class CN, class CS, int FA, int FB, int EPI, int OUT>
 __global__ __launch_bounds__(CW::THREADS) void gemm_fp8_auto_kernel(const GemmParams p) {
   static_assert(CW::BM == CN::BM && CW::THREADS == CN::THREADS, "one group table, one launch shape");
   static_assert(CN::SMEM_BYTES <= CW::SCHED_OFF, "the narrow configuration must not reach the shared group table");
   static_assert(CS::THREADS == CW::THREADS && CS::SCHED_OFF <= CW::SCHED_OFF && CS::SMEM_BYTES <= CW::SMEM_BYTES,
                 "the weight-streaming configuration shares the launch shape and must not reach the group table");
-  static_assert(CW::THREADS >= kFastMaxGroups && CW::BM == 256, "one group per thread in the count below");
+  static_assert(CW::THREADS >= kFastMaxGroups && CS::BM * 2 == CW::BM, "one group per thread; sched_init's half-height prefix is CS's");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + CW::SCHED_OFF);
-  sched_init<CW::BM>(p, sched);
+  const int32_t half_tile0 = sched_init<CW::BM>(p, sched);
   int half_full = 0;
-  if (threadIdx.x == 0) sched.pad_ = 0;
-  __syncthreads();
   if ((int)threadIdx.x < p.G) {
-    const int rows = sched.rows[threadIdx.x];
-    const int r = rows & 255;
-    half_full = r >= 1 && r <= 128;
-    const int extra = (rows + CS::BM - 1) / CS::BM - (rows + CW::BM - 1) / CW::BM;
-    if (extra) atomicAdd(&sched.pad_, extra);  // tiles that the 128-row cut has over the 256-row cut
+    const int r = sched.rows[threadIdx.x] & (CW::BM - 1);
+    half_full = r >= 1 && r <= CW::BM / 2;
   }
   const int n_half_full = __syncthreads_count(half_full);
-  const bool stream = sched.pad_ * 4 <= sched.tile0[p.G];
+  const bool stream = sched_short_tiles_pay<CW::BN>(p, sched);
   const bool narrow = sched_num_tiles<CN::BM, CN::BN>(p, sched) <= (int64_t)gridDim.x;
   const bool sit_out = n_half_full * 8 >= sched.tile0[p.G];
-  if (__builtin_expect(!narrow && !sit_out, 1))  // marked likely: the register allocator then favours this body's loops
+  if (__builtin_expect(!narrow && !stream && !sit_out, 1))  // marked likely: the register allocator then favours this body's loops
     gemm_fp8_body<CW, FA, FB, EPI, OUT, false, CW::SCHED_OFF, false>(p);
   else if (narrow)
     gemm_fp8_body<CN, FA, FB, EPI, OUT, false, CW::SCHED_OFF, true>(p);
   else if (stream) {
     if (sched.pad_ != 0) {  // some group has more than one 128-row tile: the tile prefix for this tile height
-      sched_retile<CS::BM>(p, sched);
+      sched_use_half_height(p, sched, half_tile0);
     }
-    gemm_fp8_body<CS, FA, FB, EPI, OUT, false, CW::SCHED_OFF, true>(p);
+    gemm_fp8_body<CS, FA, FB, EPI, OUT, false, CW::SCHED_OFF, false>(p);
   }
   else
     gemm_fp8_body<CW, FA, FB, EPI, OUT, false, CW::SCHED_OFF, true>(p);

@@ -16,7 +16,7 @@ struct SchedTableT {
   int64_t row0[MAXG];      // first row of the group in A/C (M modes) or first k (K modes)
   int32_t rows[MAXG];      // valid rows (M modes) or k extent (K modes)
   int32_t tile0[MAXG + 1]; // exclusive prefix of ceil(rows / BM) (M modes only)
-  int32_t pad_;            // spare word (the tuned kernels count tiles in it when they choose a configuration)
+  int32_t pad_;            // how many tiles more a cut at half the tile height has (set by sched_init)
   int64_t scan_[16];       // per-wave totals of the workgroup-wide prefix sums that build the table
 };
 typedef SchedTableT<kMaxGroups> SchedTable;
@@ -104,32 +104,26 @@ TGG_DEV int64_t sched_block_scan(int64_t v, Table& t, int64_t& total) {
   return base + inc - v;
 }
 
-// The tile prefix for another tile height BM over a table that is already built (rows do not change).
-// All threads of the workgroup must call this; G must not exceed the workgroup size; ends with a barrier.
-template <int BM, class Table>
-TGG_DEV void sched_retile(const GemmParams& p, Table& t) {
-  const int g = threadIdx.x;
-  const bool live = g < p.G;
-  int64_t total;
-  const int64_t tile0 = sched_block_scan(live ? (int64_t)((t.rows[g] + BM - 1) / BM) : 0, t, total);
-  if (live) t.tile0[g] = (int32_t)tile0;
-  if (threadIdx.x == 0) t.tile0[p.G] = (int32_t)total;
-  __syncthreads();
-}
-
 // Builds the table.  All threads of the workgroup must call this; ends with a barrier.
 // With one thread per group (G <= workgroup size <= 1024) the two prefix sums of sched_prefix -- group starts, then
 // tiles of the clipped sizes -- are workgroup-wide scans: about a microsecond, where the serial pass of one thread
 // takes 0.2 us per group (15 us at 128 groups, a tenth of a decode-sized launch).  Same values as sched_prefix.
+// The tile scan carries the prefix for tiles of half the height along in its upper word: the calling thread's group
+// would start at the returned tile id under that cut, and t.pad_ receives how many tiles more that cut has in all
+// (see sched_use_half_height).  Where the serial pass runs instead, t.pad_ is set so large that no caller prefers
+// the half-height cut.
 template <int BM, class Table>
-TGG_DEV void sched_init(const GemmParams& p, Table& t) {
+TGG_DEV int32_t sched_init(const GemmParams& p, Table& t) {
   if (p.mode == MODE_KG || p.G > (int)blockDim.x || blockDim.x > 1024) {
     for (int g = threadIdx.x; g < p.G; g += blockDim.x) sched_load_group(p, t, g);
     __syncthreads();
-    if (p.mode == MODE_KG) return;
-    if (threadIdx.x == 0) sched_prefix<BM>(p, t);
+    if (p.mode == MODE_KG) return 0;
+    if (threadIdx.x == 0) {
+      sched_prefix<BM>(p, t);
+      t.pad_ = 1 << 30;
+    }
     __syncthreads();
-    return;
+    return 0;
   }
   const int g = threadIdx.x;
   const bool live = g < p.G;
@@ -147,14 +141,30 @@ TGG_DEV void sched_init(const GemmParams& p, Table& t) {
   const int64_t limit = (p.mode == MODE_KG_COUNT) ? p.k_total : p.m_total;
   if (start >= limit) sz = 0;  // never touch rows (or k) past the end of the operands
   else if (start + sz > limit) sz = limit - start;
+  constexpr int HALF = BM / 2;
   int64_t total;
-  const int64_t tile0 = sched_block_scan((sz + BM - 1) / BM, t, total);
+  const int64_t both = sched_block_scan((sz + BM - 1) / BM + (((sz + HALF - 1) / HALF) << 32), t, total);
   if (live) {
     t.row0[g] = start;
     t.rows[g] = (int32_t)sz;
-    t.tile0[g] = (int32_t)tile0;
+    t.tile0[g] = (int32_t)(both & 0xffffffff);
   }
-  if (threadIdx.x == 0) t.tile0[p.G] = (int32_t)total;
+  if (threadIdx.x == 0) {
+    t.tile0[p.G] = (int32_t)(total & 0xffffffff);
+    t.pad_ = (int32_t)(total >> 32) - (int32_t)(total & 0xffffffff);
+  }
+  __syncthreads();
+  return (int32_t)(both >> 32);
+}
+
+// Switches a table built by sched_init<BM> to tiles of half that height: half_tile0 is what sched_init returned
+// to this thread.  All threads of the workgroup must call this; starts and ends with a barrier (other threads may
+// still be reading the totals that it overwrites).
+template <class Table>
+TGG_DEV void sched_use_half_height(const GemmParams& p, Table& t, int32_t half_tile0) {
+  __syncthreads();
+  if ((int)threadIdx.x < p.G) t.tile0[threadIdx.x] = half_tile0;
+  if (threadIdx.x == 0) t.tile0[p.G] += t.pad_;
   __syncthreads();
 }
 
@@ -177,6 +187,19 @@ TGG_HD int64_t sched_num_tiles(const GemmParams& p, const Table& t) {
     return (int64_t)p.G * tiles_m * tiles_n;
   }
   return (int64_t)t.tile0[p.G] * tiles_n;
+}
+
+// Whether tiles of half the table's tile height pay for an M-grouped launch.  t.pad_ holds the tiles that the half
+// height cut has over the table's cut (sched_init leaves it there).  The persistent workgroups work in rounds (one tile each per round), a
+// half-height tile costs about 0.7 of a full one (measured over group counts 8-256 and 64-2048 rows per group,
+// for both operand widths), and what decides is whole rounds: a launch whose full-height tiles just fit one round
+// loses by going to two rounds of short tiles, whatever their number.
+template <int BN, class Table>
+__device__ __forceinline__ bool sched_short_tiles_pay(const GemmParams& p, const Table& t) {
+  const int64_t tiles_n = (p.N + BN - 1) / BN, wgs = gridDim.x;
+  const int64_t rounds_full = ((int64_t)t.tile0[p.G] * tiles_n + wgs - 1) / wgs;
+  const int64_t rounds_half = ((int64_t)(t.tile0[p.G] + t.pad_) * tiles_n + wgs - 1) / wgs;
+  return rounds_half * 7 <= rounds_full * 10;
 }
 
 // Tile order.  Consecutive tile ids are handed to workgroups that run at the same time on one XCD
