@@ -186,9 +186,10 @@ int tgg_debug_row_tiles(const int64_t* sizes, int G, int mode, int64_t m_total, 
  *   "force_generic" 0/1  route every GEMM through the shape-agnostic kernel
  *   "variant"       int  tile configuration of the tuned kernels (16-bit, and FP8 M-grouped): 0 (default) = chosen per launch on the
  *                        device from the group sizes -- 256x128 when all such tiles fit one round of the persistent
- *                        workgroups; otherwise, 16-bit M-grouped / masked and FP8 M-grouped launches in which no group has more than
- *                        128 rows, the weight-streaming configuration (128x256 tiles, three weight slab buffers);
- *                        256x256 otherwise; 1 = always 256x128; 2 = always 256x256; 4 = always the weight-streaming
+ *                        workgroups; otherwise, for 16-bit M-grouped / masked and FP8 M-grouped launches, the
+ *                        weight-streaming configuration (128x256 tiles, three weight slab buffers) when its rounds of
+ *                        the persistent workgroups, at 0.7 of a 256-row tile's cost each, are no more than those of
+ *                        the 256x256 tiles (groups of up to about 200 rows on average); 256x256 otherwise; 1 = always 256x128; 2 = always 256x256; 4 = always the weight-streaming
  *                        configuration (16-bit NT / NN, FP8 M-grouped)
  *   "four_wave"     int  16-bit M-grouped NT: 0 (default) = eight-wave kernels, 1 = the four-wave kernel (128x128 per
  *                        wave) on large launches, 2 = on every launch it can take
