@@ -86,6 +86,40 @@ def test_m_grouped_decode_sized_groups(dev, dtype, trans_b):
     assert torch.equal(out.cpu(), gemm_ref.gmm_fp32(a, b, sizes, trans_b).to(dtype))
 
 
+def _device_choice(sizes, N, workgroups=256):
+    """The configuration that the default launch picks on the device for these group sizes: narrow tiles when all
+    of them fit one round of the workgroups; else 128-row tiles when their rounds, at 0.7 of a 256-row tile's cost,
+    are no more than the 256-row tiles' rounds; else the 256x256 tiles."""
+    t256 = sum((s + 255) // 256 for s in sizes)
+    t128 = sum((s + 127) // 128 for s in sizes)
+    if t256 * ((N + 127) // 128) <= workgroups:
+        return "narrow"
+    nb = (N + 255) // 256
+    rounds = lambda tiles: (tiles * nb + workgroups - 1) // workgroups
+    return "stream" if rounds(t128) * 7 <= rounds(t256) * 10 else "wide"
+
+
+@pytest.mark.parametrize("case", [
+    # (group sizes, N, expected choice): both sides of the rule, the 128-row cut with groups above 128 rows
+    ([200, 64, 130, 8, 0, 129, 250, 100, 256, 31] * 4, 2048, "stream"),   # 128-row cut has 1.5x the tiles, same rounds
+    ([300, 129, 257, 40, 385, 0, 130, 200] * 5, 3072, "stream"),                # three rounds against four shorter ones
+    ([512, 384, 300, 256, 700, 0, 1024, 513] * 4, 1536, "wide"),
+    ([256, 256, 255, 129] * 4, 4096, "wide"),                              # one round of 256-row tiles, two of 128-row tiles
+])
+@pytest.mark.parametrize("trans_b", [True, False])
+def test_m_grouped_device_choice_of_tile_height(dev, case, trans_b):
+    """Integer inputs through the default launch on problems that land on either side of the device-side rule
+    (mirrored in _device_choice, which also documents what each problem is meant to exercise): bit-exact against
+    the oracle, so a tile prefix that was switched to the 128-row cut wrongly would show as misplaced rows."""
+    sizes, N, want = case
+    assert _device_choice(sizes, N) == want
+    G, M, K = len(sizes), sum(sizes), 136
+    a = _ints((M, K), 21, torch.bfloat16)
+    b = _ints((G, N, K) if trans_b else (G, K, N), 22, torch.bfloat16)
+    out = m_grouped_gemm(a.to(dev), b.to(dev), torch.tensor(sizes, dtype=torch.int32, device=dev), trans_b)
+    assert torch.equal(out.cpu(), gemm_ref.gmm_fp32(a, b, sizes, trans_b).to(torch.bfloat16))
+
+
 @pytest.mark.parametrize("trans_b", [True, False])
 @pytest.mark.parametrize("sizes_dtype", [torch.int32, torch.int64])
 def test_m_grouped_random_ragged(dev, variant, trans_b, sizes_dtype):

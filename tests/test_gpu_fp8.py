@@ -246,6 +246,35 @@ def test_fp8_block_scaled_exact_with_power_of_two_scales(dev, variant, K):
         start += p
 
 
+@pytest.mark.parametrize("sizes,N", [
+    ([200, 64, 130, 8, 0, 129, 250, 100, 256, 31] * 4, 2048),    # the device picks 128-row tiles; groups above 128 rows
+    ([300, 129, 257, 40, 385, 0, 130, 200] * 5, 3072),           # likewise, three rounds against four shorter ones
+    ([512, 384, 300, 256, 700, 0, 1024, 513] * 4, 1536),         # 256-row tiles
+])
+def test_fp8_block_scaled_device_choice_of_tile_height(dev, sizes, N):
+    """The default launch on problems on either side of the device-side choice of tile height (the same rule as in
+    the 16-bit kernels, see test_gpu_bf16._device_choice): small-integer codes and power-of-two scales, so the
+    result must equal the closed form bit for bit; a tile prefix switched to the 128-row cut wrongly, or scales
+    fetched for the wrong rows, would show."""
+    g = torch.Generator().manual_seed(71)
+    padded = [(s + 127) // 128 * 128 for s in sizes]
+    Mp, G, K = sum(padded), len(sizes), 256
+    aq = torch.randint(-3, 4, (Mp, K), generator=g).float()
+    bq = torch.randint(-3, 4, (G, N, K), generator=g).float()
+    pw = torch.tensor([0.25, 0.5, 1.0, 2.0])
+    sa = pw[torch.randint(0, 4, (Mp, K // 128), generator=g)]
+    sb = pw[torch.randint(0, 4, (G, N // 128, K // 128), generator=g)]
+    out = m_grouped_fp8_nt_contiguous((aq.to(torch.float8_e4m3fn).to(dev), sa.to(dev)),
+                                      (bq.to(torch.float8_e4m3fn).to(dev), sb.to(dev)),
+                                      torch.tensor(sizes, dtype=torch.int32, device=dev))
+    ref = gemm_ref.fp8_block_scaled_reference(aq, sa, bq, sb, sizes).to(torch.bfloat16)
+    out = out.cpu()
+    start = 0
+    for s_, p_ in zip(sizes, padded):
+        assert torch.equal(out[start:start + s_], ref[start:start + s_])
+        start += p_
+
+
 def test_fp8_block_scaled_per_row_layout_in_any_expert_order(dev, variant):
     """Experts' regions in a shuffled order, stated by a per-row layout (gemm/deep_gemm_ops.py:60-100 forwards any):
     small-integer codes and power-of-two scales, so the closed form is exact; checked row by row from the layout."""
