@@ -110,3 +110,37 @@ def test_group_sizes_may_change_between_replays(dev):
         exact = ad @ wd.t()
         assert float((out8[:n0].float() - exact).abs().max()) <= 2.0 ** -7 * float(exact.abs().max()), f"replay {it} (fp8 values)"
         assert bool((out16[rows:] == 7.0).all()) and bool((out8[placed:] == 7.0).all()), f"replay {it}: rows past the groups"
+
+
+def test_deep_gemm_shaped_wrappers_can_be_captured(dev):
+    """m_grouped_bf16_nt_contiguous / m_grouped_fp8_nt_contiguous check M against the padded sizes on the host, as
+    the reference does; under capture that read is left out, so the wrappers themselves can sit in a graph (with
+    ``out=`` given).  Replays must equal the eager calls."""
+    from triton_grouped_gemm_amd.gemm.deep_gemm_ops import m_grouped_bf16_nt_contiguous, m_grouped_fp8_nt_contiguous
+    from triton_grouped_gemm_amd.quant.fp8_cast import per_block_cast_to_fp8, per_token_cast_to_fp8
+    sizes_list = [100, 0, 256, 31, 128, 385]
+    padded = [(s + 127) // 128 * 128 for s in sizes_list]
+    G, M, N, K = len(sizes_list), sum(padded), 512, 256
+    sizes = torch.tensor(sizes_list, dtype=torch.int32, device=dev)
+    a, b = _randn((M, K), 31, dev), _randn((G, N, K), 32, dev)
+    aq = per_token_cast_to_fp8(a, scales_mn_major=True)
+    wq = per_block_cast_to_fp8(b)
+    out16 = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+    out8 = torch.zeros((M, N), dtype=torch.bfloat16, device=dev)
+    ref16 = m_grouped_bf16_nt_contiguous(a, b, sizes, out=torch.zeros_like(out16))
+    ref8 = m_grouped_fp8_nt_contiguous(aq, wq, sizes, out=torch.zeros_like(out8))
+    with pytest.raises(ValueError):  # eagerly the reference's check stays
+        m_grouped_bf16_nt_contiguous(a[:-128], b, sizes)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        m_grouped_bf16_nt_contiguous(a, b, sizes, out=out16)
+        m_grouped_fp8_nt_contiguous(aq, wq, sizes, out=out8)
+    for it in range(3):
+        out16.zero_()
+        out8.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out16, ref16), f"replay {it}"
+        assert torch.equal(out8, ref8), f"replay {it} (fp8)"
