@@ -190,10 +190,10 @@ TGG_HD int64_t sched_num_tiles(const GemmParams& p, const Table& t) {
 }
 
 // Whether tiles of half the table's tile height pay for an M-grouped launch.  t.pad_ holds the tiles that the half
-// height cut has over the table's cut (sched_init leaves it there).  The persistent workgroups work in rounds (one tile each per round), a
-// half-height tile costs about 0.7 of a full one (measured over group counts 8-256 and 64-2048 rows per group,
-// for both operand widths), and what decides is whole rounds: a launch whose full-height tiles just fit one round
-// loses by going to two rounds of short tiles, whatever their number.
+// height cut has over the table's cut (sched_init leaves it there).  The persistent workgroups work in rounds (one
+// tile each per round), a half-height tile costs about 0.7 of a full one (measured over group counts 8-256 and
+// 64-2048 rows per group, for both operand widths), and what decides is whole rounds: a launch whose full-height
+// tiles just fit one round loses by going to two rounds of short tiles, whatever their number.
 template <int BN, class Table>
 __device__ __forceinline__ bool sched_short_tiles_pay(const GemmParams& p, const Table& t) {
   const int64_t tiles_n = (p.N + BN - 1) / BN, wgs = gridDim.x;
