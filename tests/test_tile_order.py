@@ -95,6 +95,26 @@ def test_k_grouped_cover(tile, grid):
     assert n == len(exp) and set(got) == exp and len(set(got)) == len(got)
 
 
+def test_k_grouped_tile_space_runs_over_groups_by_decreasing_size():
+    """A K-grouped tile costs what its group has tokens and every group has equally many tiles, so the tile space
+    lists the groups by decreasing token count (ties by index): with a fixed stride every workgroup then sees a
+    fair mix, and the launch ends on its cheapest tiles."""
+    sizes, mdim, N = [40, 0, 200, 64, 200, 8, 0, 512], 256, 512
+    rows, n = tile_order(sizes, KG_COUNT, mdim, sum(sizes), N, 256, 1, 0)  # one workgroup: it walks the ids in order
+    per_group = 2
+    assert n == len(sizes) * per_group
+    walked = [int(r[2]) for r in rows.tolist()]
+    want = sorted(range(len(sizes)), key=lambda g: (-sizes[g], g))
+    assert walked == [g for g in want for _ in range(per_group)]
+    # the loads of 4 workgroups that take every fourth tile: within one largest group of each other
+    sizes = [(37 * g * g + 11 * g) % 2000 for g in range(64)]
+    rows, n = tile_order(sizes, KG_COUNT, 256, sum(sizes), 768, 256, 4, 0)  # 3 tiles per group, grid of 4
+    load = [0] * 4
+    for b, _, g, *_ in rows.tolist():
+        load[int(b)] += sizes[int(g)]
+    assert max(load) - min(load) <= max(sizes)
+
+
 def test_runs_of_an_xcd_are_near_square():
     """With 256 workgroups dealt round robin to 8 XCDs, the 32 tiles an XCD works on at the same time should
     span few distinct row panels and column panels (this is what keeps operand re-reads inside one L2)."""

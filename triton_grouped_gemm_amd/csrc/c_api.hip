@@ -94,6 +94,7 @@ static int tile_order_host(const GemmParams& p, int grid, int split, int64_t* ou
   SchedTable* t = new SchedTable;
   for (int g = 0; g < p.G; ++g) sched_load_group(p, *t, g);
   sched_prefix<BM>(p, *t);
+  if (p.mode == MODE_KG || p.mode == MODE_KG_COUNT) sched_order_groups_serial(p, *t);
   const int64_t total = sched_num_tiles<BM, BN>(p, *t);
   *num_tiles = total;
   int64_t n = 0;

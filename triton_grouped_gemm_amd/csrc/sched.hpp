@@ -15,7 +15,7 @@ template <int MAXG>
 struct SchedTableT {
   int64_t row0[MAXG];      // first row of the group in A/C (M modes) or first k (K modes)
   int32_t rows[MAXG];      // valid rows (M modes) or k extent (K modes)
-  int32_t tile0[MAXG + 1]; // exclusive prefix of ceil(rows / BM) (M modes only)
+  int32_t tile0[MAXG + 1]; // M modes: exclusive prefix of ceil(rows / BM); K modes: the groups in the order of the tile space (sched_order_groups)
   int32_t pad_;            // how many tiles more a cut at half the tile height has (set by sched_init)
   int64_t scan_[16];       // per-wave totals of the workgroup-wide prefix sums that build the table
 };
@@ -80,6 +80,29 @@ TGG_HD void sched_prefix(const GemmParams& p, Table& t) {
   t.tile0[G] = tile;
 }
 
+// K-grouped tile space: a tile costs what its group has tokens, every group has the same number of tiles, and the
+// persistent workgroups take tile ids with a fixed stride -- so with 192 tiles per group and 256 workgroups each
+// workgroup misses every fourth group, and which fourth decides its load.  The tile space therefore runs over the
+// groups in order of decreasing token count (ties by index): the sums over every fourth group of a sorted sequence
+// differ by less than the largest group, and the launch ends on its cheapest tiles.  t.tile0[i] = the group whose
+// tiles come i-th.  Position of group g = number of groups that precede it in that order.
+template <class Table>
+TGG_HD int sched_group_rank(const Table& t, int G, int g) {
+  const int32_t mine = t.rows[g];
+  int rank = 0;
+  for (int h = 0; h < G; ++h) {
+    const int32_t other = t.rows[h];
+    rank += (other > mine) || (other == mine && h < g);
+  }
+  return rank;
+}
+
+// Serial form (host hook, and kernels whose workgroups have fewer threads than there are groups).
+template <class Table>
+TGG_HD void sched_order_groups_serial(const GemmParams& p, Table& t) {
+  for (int g = 0; g < p.G; ++g) t.tile0[sched_group_rank(t, p.G, g)] = g;
+}
+
 // Exclusive prefix sum over the workgroup's threads (in thread order) and the total; all threads must call it.
 // Wave-wide scan by lane exchange, the waves' totals through the table's scratch words.
 template <class Table>
@@ -104,6 +127,15 @@ TGG_DEV int64_t sched_block_scan(int64_t v, Table& t, int64_t& total) {
   return base + inc - v;
 }
 
+// K modes only (a no-op otherwise): fills t.tile0 with the groups in tile-space order once t.rows is final.  All
+// threads of the workgroup must call this; ends with a barrier when it does anything.
+template <class Table>
+TGG_DEV void sched_order_groups(const GemmParams& p, Table& t) {
+  if (p.mode != MODE_KG && p.mode != MODE_KG_COUNT) return;
+  for (int g = threadIdx.x; g < p.G; g += blockDim.x) t.tile0[sched_group_rank(t, p.G, g)] = g;
+  __syncthreads();
+}
+
 // Builds the table.  All threads of the workgroup must call this; ends with a barrier.
 // With one thread per group (G <= workgroup size <= 1024) the two prefix sums of sched_prefix -- group starts, then
 // tiles of the clipped sizes -- are workgroup-wide scans: about a microsecond, where the serial pass of one thread
@@ -117,12 +149,14 @@ TGG_DEV int32_t sched_init(const GemmParams& p, Table& t) {
   if (p.mode == MODE_KG || p.G > (int)blockDim.x || blockDim.x > 1024) {
     for (int g = threadIdx.x; g < p.G; g += blockDim.x) sched_load_group(p, t, g);
     __syncthreads();
-    if (p.mode == MODE_KG) return 0;
-    if (threadIdx.x == 0) {
-      sched_prefix<BM>(p, t);
-      t.pad_ = 1 << 30;
+    if (p.mode != MODE_KG) {
+      if (threadIdx.x == 0) {
+        sched_prefix<BM>(p, t);
+        t.pad_ = 1 << 30;
+      }
+      __syncthreads();
     }
-    __syncthreads();
+    sched_order_groups(p, t);
     return 0;
   }
   const int g = threadIdx.x;
@@ -154,6 +188,7 @@ TGG_DEV int32_t sched_init(const GemmParams& p, Table& t) {
     t.pad_ = (int32_t)(total >> 32) - (int32_t)(total & 0xffffffff);
   }
   __syncthreads();
+  sched_order_groups(p, t);
   return (int32_t)(both >> 32);
 }
 
@@ -273,9 +308,10 @@ TGG_HD Tile sched_tile(const GemmParams& p, const Table& t, int64_t tile_id, int
   if (p.mode == MODE_KG || p.mode == MODE_KG_COUNT) {
     const int tiles_m = (int)((p.m_total + BM - 1) / BM);
     const int per_group = tiles_m * tiles_n;
-    r.g = tid32 / per_group;
+    const int slot = tid32 / per_group;
+    r.g = t.tile0[slot];  // groups in order of decreasing size, see sched_group_rank
     int mt, nt;
-    sched_split(tid32 - r.g * per_group, tiles_m, tiles_n, nc, mt, nt);
+    sched_split(tid32 - slot * per_group, tiles_m, tiles_n, nc, mt, nt);
     r.n0 = nt * BN;
     r.row0 = (int64_t)mt * BM;
     const int64_t left = p.m_total - r.row0;
