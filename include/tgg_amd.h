@@ -61,6 +61,18 @@ int tgg_m_grouped_gemm_masked(const void* A, const void* B, void* C, const void*
 int tgg_k_grouped_gemm(const void* A, const void* B, void* C, const int32_t* start, const int32_t* end, int G,
                        int Mdim, int N, int64_t Ktot, int dtype, int num_cu, void* stream);
 
+/* tgg_k_grouped_gemm with a work queue (same reference function, gemm/BF16/k_grouped_gemm_TMA.py:217-294).  A
+ * K-grouped tile costs what its group has tokens, so with ragged groups no fixed assignment of tiles to the
+ * persistent workgroups is even.  `queue` points to TGG_QUEUE_WORDS int32 in device memory that are ZERO when the
+ * kernel starts (clear them on the same stream, with a fill kernel if the call may be captured into a graph); the
+ * workgroups draw their tile ids from them (one counter per XCD), largest groups first, and a workgroup that drew
+ * expensive tiles draws fewer.  Results are bit-identical to tgg_k_grouped_gemm; the kernel leaves the counters at
+ * the numbers of ids drawn.  A launch must have the words to itself until it has finished.  queue = NULL: the
+ * fixed assignment. */
+#define TGG_QUEUE_WORDS 8
+int tgg_k_grouped_gemm_queued(const void* A, const void* B, void* C, const int32_t* start, const int32_t* end, int G,
+                              int Mdim, int N, int64_t Ktot, int dtype, int num_cu, int32_t* queue, void* stream);
+
 /* C = (Aq . Bq[g]^T) * a_scale[r] * b_scale[g*N+n].  Replaces gmm_fp8_act_per_channel_w_per_expert
  * (gemm/FP8/m_grouped_gemm_channel_expert.py:139-198). */
 int tgg_m_grouped_gemm_fp8_channel(const void* Aq, const float* a_scale, const void* Bq, const float* b_scale,
@@ -74,6 +86,13 @@ int tgg_m_grouped_gemm_fp8_channel(const void* Aq, const float* a_scale, const v
 int tgg_k_grouped_gemm_fp8_channel(const void* x, const float* xs, const void* y, const float* ys, void* out,
                                    const int32_t* tokens, int G, int M, int N, int64_t Ktot, int fmt_a, int fmt_b,
                                    int num_cu, void* stream);
+
+/* tgg_k_grouped_gemm_fp8_channel with a work queue (same reference function,
+ * gemm/FP8/k_grouped_gemm_channel_expert.py:143-181); `queue` as in tgg_k_grouped_gemm_queued.  Only the tuned
+ * kernel (token counts that are all multiples of 16) draws from it; the shape-agnostic kernel leaves it untouched. */
+int tgg_k_grouped_gemm_fp8_channel_queued(const void* x, const float* xs, const void* y, const float* ys, void* out,
+                                          const int32_t* tokens, int G, int M, int N, int64_t Ktot, int fmt_a,
+                                          int fmt_b, int num_cu, int32_t* queue, void* stream);
 
 /* out[r,n] = sum_kb (sum_{k in kb} Aq[r,k] Bq[g,n,k]) * sa[r,kb] * sb[g,n/128,kb]; e4m3fn codes, A physically
  * padded per group to `align` rows, sb [G,ceil(N/128),ceil(K/128)], bf16 output.  sa holds M x ceil(K/128)

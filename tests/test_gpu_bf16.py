@@ -362,3 +362,35 @@ def test_many_groups_exact(dev, variant, G):
     kt = k_grouped_gemm(a.to(dev), a.to(dev), torch.tensor(sizes, dtype=torch.int64, device=dev))
     ref = gemm_ref.gmm_dw(a, a, sizes, fp32=True)
     assert ref.abs().max() <= 256 and torch.equal(kt.cpu(), ref.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("sizes", [
+    [5000, 0, 64, 1200, 0, 0, 8, 300, 2048, 16, 700, 1],      # few long tiles, runs of empty and one-slab groups
+    [64] * 40,                                                # one-slab tiles only: the copy stream looks furthest ahead
+    [0, 0, 0, 9000],                                          # empty groups first in index order
+    [(53 * g * g + 17 * g) % 3000 for g in range(96)],
+])
+def test_k_grouped_work_queue_equals_fixed_assignment(dev, sizes):
+    """tgg_k_grouped_gemm_queued (tile ids drawn from counters in device memory, largest groups first) against
+    tgg_k_grouped_gemm (fixed assignment) and the oracle: same bits, whichever workgroup computes a tile; the
+    counters end at the number of draws, at least one per tile."""
+    from triton_grouped_gemm_amd import _native
+    G, Mdim, N = len(sizes), 520, 776
+    Kt = sum(sizes)
+    a, b = _randn((Kt, Mdim), 1.0, 31).to(dev), _randn((Kt, N), 1.0, 32).to(dev)
+    s = torch.tensor(sizes, dtype=torch.int32, device=dev)
+    end = s.cumsum(0).to(torch.int32)
+    start = (end - s).to(torch.int32)
+    fixed = torch.full((G, Mdim, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    drawn = torch.full((G, Mdim, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    queue = torch.zeros(_native.QUEUE_WORDS, dtype=torch.int32, device=dev)
+    st = _native.stream_of(a)
+    _native.call("tgg_k_grouped_gemm", a.data_ptr(), b.data_ptr(), fixed.data_ptr(), start.data_ptr(), end.data_ptr(),
+                 G, Mdim, N, Kt, _native.BF16, -1, st)
+    _native.call("tgg_k_grouped_gemm_queued", a.data_ptr(), b.data_ptr(), drawn.data_ptr(), start.data_ptr(),
+                 end.data_ptr(), G, Mdim, N, Kt, _native.BF16, -1, queue.data_ptr(), st)
+    assert torch.equal(fixed, drawn)
+    tiles = G * ((Mdim + 255) // 256) * ((N + 255) // 256)
+    assert int(queue.sum()) >= tiles
+    check_16bit_gemm(drawn, gemm_ref.gmm_dw(a.cpu(), b.cpu(), sizes), gemm_ref.gmm_dw(a.cpu(), b.cpu(), sizes, fp32=True),
+                     "queued K-grouped")

@@ -183,6 +183,33 @@ def test_fp8_channel_k_grouped_unpadded_counts(dev, tokens, tuned_runs, M, N):
         assert torch.equal(outs["default"], outs["generic"])  # ... to the shape-agnostic kernel
 
 
+@pytest.mark.parametrize("tokens", [[512, 0, 128, 2048, 16, 0, 0, 640, 128, 128, 1024, 16], [128] * 24])
+def test_fp8_k_grouped_work_queue_equals_fixed_assignment(dev, tokens):
+    """tgg_k_grouped_gemm_fp8_channel_queued (tile ids drawn from counters in device memory) against the fixed
+    assignment: same bits whichever workgroup computes a tile.  Token counts are multiples of 16, so the tuned
+    kernel runs and draws; the wrapper's own result (queued as well) is checked against the oracle elsewhere."""
+    from triton_grouped_gemm_amd import _native
+    M, N, G = 264, 520, len(tokens)
+    xq, xs, yq, ys = _k_grouped_unpadded_case(tokens, M, N, 90)
+    Kt = sum(tokens)
+    x = _codes_to_torch(xq, "e4m3fn").contiguous().to(dev)
+    y = _codes_to_torch(yq, "e4m3fn").contiguous().to(dev)
+    xs_t = torch.from_numpy(np.ascontiguousarray(xs.T)).to(dev)  # element (row, g) at g * rows + row
+    ys_t = torch.from_numpy(np.ascontiguousarray(ys.T)).to(dev)
+    tok = torch.tensor(tokens, dtype=torch.int32, device=dev)
+    fixed = torch.full((G, M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    drawn = torch.full((G, M, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    queue = torch.zeros(_native.QUEUE_WORDS, dtype=torch.int32, device=dev)
+    st = _native.stream_of(x)
+    _native.call("tgg_k_grouped_gemm_fp8_channel", x.data_ptr(), xs_t.data_ptr(), y.data_ptr(), ys_t.data_ptr(),
+                 fixed.data_ptr(), tok.data_ptr(), G, M, N, Kt, _native.E4M3, _native.E4M3, -1, st)
+    _native.call("tgg_k_grouped_gemm_fp8_channel_queued", x.data_ptr(), xs_t.data_ptr(), y.data_ptr(), ys_t.data_ptr(),
+                 drawn.data_ptr(), tok.data_ptr(), G, M, N, Kt, _native.E4M3, _native.E4M3, -1, queue.data_ptr(), st)
+    assert not bool(torch.isnan(fixed.float()).any())
+    assert torch.equal(fixed, drawn)
+    assert int(queue.sum()) >= G * ((M + 255) // 256) * ((N + 255) // 256)
+
+
 def _block_scaled_case(sizes, N, K, seed):
     padded = [(s + 127) // 128 * 128 for s in sizes]
     Mp, G = sum(padded), len(sizes)

@@ -15,6 +15,7 @@ LIB_PATH = Path(__file__).resolve().parent / "libtgg_amd.so"
 
 BF16, F16, E4M3, E5M2 = 0, 1, 2, 3
 MAX_GROUPS = 1024
+QUEUE_WORDS = 8  # TGG_QUEUE_WORDS: int32 counters of the K-grouped kernels' work queue
 
 _P, _I, _L = c_void_p, c_int, c_int64
 
@@ -25,8 +26,10 @@ SIGNATURES = {
     "tgg_m_grouped_gemm_placed": [_P, _P, _P, _P, _I, _P, _I, _L, _I, _I, _I, _I, _P],
     "tgg_m_grouped_gemm_masked": [_P, _P, _P, _P, _I, _I, _L, _L, _I, _I, _I, _I, _I, _P],
     "tgg_k_grouped_gemm": [_P, _P, _P, _P, _P, _I, _I, _I, _L, _I, _I, _P],
+    "tgg_k_grouped_gemm_queued": [_P, _P, _P, _P, _P, _I, _I, _I, _L, _I, _I, _P, _P],
     "tgg_m_grouped_gemm_fp8_channel": [_P, _P, _P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _I, _I, _P],
     "tgg_k_grouped_gemm_fp8_channel": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _L, _I, _I, _I, _P],
+    "tgg_k_grouped_gemm_fp8_channel_queued": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _L, _I, _I, _I, _P, _P],
     "tgg_m_grouped_gemm_fp8_block": [_P, _P, _P, _P, _P, _P, _I, _I, _L, _I, _I, _I, _I, _I, _P],
     "tgg_m_grouped_gemm_fp8_block_placed": [_P, _P, _P, _P, _P, _P, _I, _P, _I, _L, _I, _I, _I, _I, _P],
     "tgg_trans_per_block_quant_expand_128x": [_P, _P, _P, _P, _I, _I, _L, _I, _L, _I, _P],

@@ -220,6 +220,11 @@ int tgg_m_grouped_gemm_masked(const void* A, const void* B, void* C, const void*
 
 int tgg_k_grouped_gemm(const void* A, const void* B, void* C, const int32_t* start, const int32_t* end, int G,
                        int Mdim, int N, int64_t Ktot, int dtype, int num_cu, void* stream) {
+  return tgg_k_grouped_gemm_queued(A, B, C, start, end, G, Mdim, N, Ktot, dtype, num_cu, nullptr, stream);
+}
+
+int tgg_k_grouped_gemm_queued(const void* A, const void* B, void* C, const int32_t* start, const int32_t* end, int G,
+                              int Mdim, int N, int64_t Ktot, int dtype, int num_cu, int32_t* queue, void* stream) {
   if (int e = check_common(A, B, C, start, G, N)) return e;
   if (!end) return set_error("null group_end pointer");
   if (Mdim < 1 || Ktot < 0) return set_error("bad Mdim=%d or Ktot=%lld", Mdim, (long long)Ktot);
@@ -230,6 +235,7 @@ int tgg_k_grouped_gemm(const void* A, const void* B, void* C, const int32_t* sta
   p.mode = MODE_KG; p.m_total = Mdim; p.k_total = Ktot; p.N = N; p.K = 0;
   p.a_sm = 1; p.a_sk = Mdim; p.b_sg = 0; p.b_sn = 1; p.b_sk = N; p.c_sg = (int64_t)Mdim * N;
   p.grid_limit = num_cu;
+  p.queue = queue;
   return dispatch_16bit(p, dtype, 2, (hipStream_t)stream);
 }
 
@@ -257,6 +263,12 @@ int tgg_m_grouped_gemm_fp8_channel(const void* Aq, const float* a_scale, const v
 int tgg_k_grouped_gemm_fp8_channel(const void* x, const float* xs, const void* y, const float* ys, void* out,
                                    const int32_t* tokens, int G, int M, int N, int64_t Ktot, int fmt_a, int fmt_b,
                                    int num_cu, void* stream) {
+  return tgg_k_grouped_gemm_fp8_channel_queued(x, xs, y, ys, out, tokens, G, M, N, Ktot, fmt_a, fmt_b, num_cu, nullptr, stream);
+}
+
+int tgg_k_grouped_gemm_fp8_channel_queued(const void* x, const float* xs, const void* y, const float* ys, void* out,
+                                          const int32_t* tokens, int G, int M, int N, int64_t Ktot, int fmt_a,
+                                          int fmt_b, int num_cu, int32_t* queue, void* stream) {
   if (int e = check_common(x, y, out, tokens, G, N)) return e;
   if (!xs || !ys) return set_error("null scale pointer");
   if (M < 1 || Ktot < 0) return set_error("bad M=%d or Ktot=%lld", M, (long long)Ktot);
@@ -268,6 +280,7 @@ int tgg_k_grouped_gemm_fp8_channel(const void* x, const float* xs, const void* y
   p.mode = MODE_KG_COUNT; p.m_total = M; p.k_total = Ktot; p.N = N; p.K = 0;
   p.a_sm = Ktot; p.a_sk = 1; p.b_sg = 0; p.b_sn = Ktot; p.b_sk = 1; p.c_sg = (int64_t)M * N;
   p.grid_limit = num_cu;
+  p.queue = queue;
   if (!g_force_generic && fast_fp8_supported(p, false)) {
     // The tuned kernel needs every token count to be a multiple of 16 and only the device knows the counts: both
     // kernels are enqueued, each reads the counts first and exactly one of them runs (the other returns at once).

@@ -97,6 +97,7 @@ struct GemmParams {
   int grid_limit;         // >0 caps the persistent grid
   int tile_split;         // tuned kernels: 1 = per-XCD contiguous tile ranges (see sched_walk)
   int n_chunk;            // column tiles per chunk of the tile order, 0 = automatic (see sched_tile)
+  int32_t* queue;         // K-grouped tuned kernels: tile-id counter in device memory (zero at launch), or null = static walk
   int store_nt;           // tuned kernels: 1 = non-temporal output stores
   // FP8 K-grouped by token counts: the tuned kernel copies 16-byte chunks, so it needs every count (hence every
   // segment start) to be a multiple of 16; the shape-agnostic kernel takes anything.  Only the device knows the

@@ -105,7 +105,8 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
   typedef Operand<C::BN, B_KMAJOR> OpB;
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  const auto& sched = *reinterpret_cast<const SchedTableT<kFastMaxGroups>*>(smem + SCHED_AT);
+  auto& sched_rw = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + SCHED_AT);
+  const auto& sched = sched_rw;
   const int64_t num_tiles = sched_num_tiles<C::BM, C::BN>(p, sched);
 
   const uint32_t smem_addr = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
@@ -187,8 +188,13 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
   };
   const int64_t a_step = A_KMAJOR ? BK * 2 : BK * a_ld;
   const int64_t b_step = B_KMAJOR ? BK * 2 : BK * b_ld;
+  // Queued launches (see tile_at below) give the tiles of an empty group one slab of nothing instead of none: the
+  // copy stream then advances by exactly one tile per tile, which bounds how far ahead of the multiplies it looks.
+  const bool queued = LAYOUT == LAYOUT_TN && p.queue != nullptr;
   auto slabs_of = [&](const Tile& t) -> int {
-    return LAYOUT == LAYOUT_TN ? (int)((t.k1 - t.k0 + BK - 1) / BK) : (p.K + BK - 1) / BK;
+    if (LAYOUT != LAYOUT_TN) return (p.K + BK - 1) / BK;
+    const int n = (int)((t.k1 - t.k0 + BK - 1) / BK);
+    return queued && n == 0 ? 1 : n;
   };
   auto make_io = [&](const Tile& t) {
     TileIo io;
@@ -234,26 +240,66 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
   // being multiplied.  Once the sequence is exhausted the descriptors get length zero: nothing is
   // fetched, but every wave still issues the same number of copies, which keeps the waits uniform.
   const TileWalk walk = sched_walk(num_tiles, LAYOUT != LAYOUT_TN && p.tile_split);
+  // The workgroup's pos-th tile (-1 past its last one).  Static: the walk above.  Queued (K-grouped, whose tiles
+  // cost what their groups have tokens, with the groups in order of decreasing size): tile ids are drawn from a
+  // counter in global memory, so a workgroup that drew expensive tiles simply draws fewer -- the greedy schedule
+  // that evens out what no fixed assignment can.  Thread 0 draws and passes the ids to the other waves through a
+  // ring of eight words in the group table's scan scratch; readers use plain LDS reads, so an id must be drawn a
+  // workgroup barrier before anyone can ask for it.  Who asks first is the copy stream: it runs two slabs ahead of
+  // the multiplies and looks the next tile up as soon as it has requested a tile's last slab.  Thread 0 draws once
+  // per tile, right after the barrier of the tile's first slab (what it writes there is seen by all from the
+  // second slab after that one on), and draws on through short tiles until it has drawn one of at least
+  // kLongTile slabs -- that one gives the next draw time enough -- or is kQueueAhead tiles ahead (enough for any
+  // run of one-slab tiles).  So a workgroup commits itself to one expensive tile beyond the one in work, not more:
+  // committing to several is what spoils the balance when a workgroup has only a dozen tiles in all.  Ids at or
+  // beyond the tile count end the workgroup's sequence; the counter only grows, so all later ones are too.
+  constexpr int kQueueAhead = 5, kLongTile = 5;
+  int32_t* const qring = reinterpret_cast<int32_t*>(sched_rw.scan_);
+  const int total_tiles = (int)num_tiles;
+  auto tile_at = [&](int pos) -> int {
+    if (queued) {
+      const int id = __builtin_amdgcn_readfirstlane(qring[pos & 7]);
+      return id < total_tiles ? id : -1;
+    }
+    const int64_t id = walk.first + (int64_t)pos * walk.stride;
+    return id < walk.end ? (int)id : -1;
+  };
+  int q_drawn = 0, q_victim = 0;  // thread 0: ids drawn so far, counters found exhausted (see sched_draw_tile)
+  // thread 0: makes sure the ids of tiles from..from+kQueueAhead-1 are drawn, up to the first long tile
+  auto draw_from = [&](int from) {
+    for (int j = from; j < from + kQueueAhead; ++j) {
+      if (j >= q_drawn) {
+        qring[j & 7] = sched_draw_tile(p.queue, total_tiles, q_victim);
+        ++q_drawn;
+      }
+      const int id = qring[j & 7];
+      if (id >= total_tiles || slabs_of(sched_tile<C::BM, C::BN>(p, sched, id)) >= kLongTile) break;
+    }
+  };
+  if (queued) {
+    if (threadIdx.x == 0) draw_from(0);
+    __syncthreads();
+  }
   TileIo feed;
-  int64_t feed_id;
+  int feed_pos = 0;
   // The tile the feed last looked up is kept: it is the one the multiplying loop asks for a little later, which
   // saves that loop the lookup (a chain of dependent LDS reads right before a tile's first multiplies).
   Tile seen;
-  int64_t seen_id = -1;
+  int seen_id = -1;
   int seen_g = -1;
   // DEEP: the B copies have a cursor of their own, one slab ahead of `feed` (which then serves A only); it does
   // the tile lookups and `feed` reuses them.
   TileIo feedb;
-  int64_t feedb_id = -1;
+  int feedb_pos = 0;
   Tile seenb;
-  int64_t seenb_id = -1;
+  int seenb_id = -1;
   int seenb_g = -1;
-  auto feedb_seek = [&](int64_t id) {
+  auto feedb_seek = [&](int pos) {
     feedb.kt_n = 0;
     feedb.issued = 0;
     feedb.a_base = feedb.b_base = (uint64_t)p.A;
     feedb.a_rem = feedb.b_rem = feedb.a_off = feedb.b_off = 0;
-    for (; id < walk.end; id += walk.stride) {
+    for (int id; (id = tile_at(pos)) >= 0; ++pos) {
       const Tile tt = sched_tile<C::BM, C::BN>(p, sched, id, seenb_g);
       seenb = tt;
       seenb_id = id;
@@ -263,14 +309,14 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
         break;
       }
     }
-    feedb_id = id;
+    feedb_pos = pos;
   };
-  auto feed_seek = [&](int64_t id) {
+  auto feed_seek = [&](int pos) {
     feed.kt_n = 0;
     feed.issued = 0;
     feed.a_base = feed.b_base = (uint64_t)p.A;
     feed.a_rem = feed.b_rem = feed.a_off = feed.b_off = 0;
-    for (; id < walk.end; id += walk.stride) {
+    for (int id; (id = tile_at(pos)) >= 0; ++pos) {
       const Tile tt = (DEEP && id == seenb_id) ? seenb : sched_tile<C::BM, C::BN>(p, sched, id, seen_g);
       seen = tt;
       seen_id = id;
@@ -280,7 +326,7 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
         break;
       }
     }
-    feed_id = id;
+    feed_pos = pos;
   };
   // One slab's copies are requested in two halves, interleaved with multiplies (see the pipeline below):
   // begin_slab fixes the descriptors and moves the feed on, copy_k issues this wave's k-th copy.
@@ -307,12 +353,14 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
     feedb.b_base += b_step;
     feedb.b_rem -= B_KMAJOR ? BK * 2 : BK;
     feedb.issued += 1;
-    if (live && feedb.issued >= feedb.kt_n) feedb_seek(feedb_id + walk.stride);
+    if (live && feedb.issued >= feedb.kt_n) feedb_seek(feedb_pos + 1);
   };
   // buf: the A buffer (and, with two B buffers, the B buffer); buf_b: the B buffer of the deep ring
   auto begin_slab = [&](int buf, int buf_b = 0) {
     SlabCopy sc;
-    const bool live = feed.issued < feed.kt_n;
+    const bool counted = feed.issued < feed.kt_n;
+    // a queued launch's slab of nothing (empty group): counted like any slab, fetches nothing
+    const bool live = counted && (LAYOUT != LAYOUT_TN || feed.a_rem > 0);
     const int a_len = A_KMAJOR ? feed.a_rem : min(feed.a_rem, BK) * (int)a_ld - feed.a_off;
     const int b_len = B_KMAJOR ? feed.b_rem : min(feed.b_rem, BK) * (int)b_ld - feed.b_off;
     sc.ra = make_rsrc32(feed.a_base, live ? a_len : 0);
@@ -328,7 +376,7 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
     feed.b_base += b_step;
     feed.b_rem -= B_KMAJOR ? BK * 2 : BK;
     feed.issued += 1;
-    if (live && feed.issued >= feed.kt_n) feed_seek(feed_id + walk.stride);
+    if (counted && feed.issued >= feed.kt_n) feed_seek(feed_pos + 1);
     if (DEEP) begin_b(sc, buf_b);
     return sc;
   };
@@ -359,8 +407,8 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
   // DEEP: per slab r the A copies of slab r+2 and then the B copies of slab r+3 are issued; the wait in slab r+1
   // lets the most recent CB copies (those B copies) stay in flight: loads complete in order, so all older ones are done.
   constexpr int WAIT_N = DEEP ? CB : 0;
-  if (DEEP) feedb_seek(walk.first);
-  feed_seek(walk.first);
+  if (DEEP) feedb_seek(0);
+  feed_seek(0);
   {
     SlabCopy s0 = begin_slab(0, 0);
 #pragma unroll
@@ -402,7 +450,7 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
       for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
   };
 
-  for (int64_t tile_id = walk.first; tile_id < walk.end; tile_id += walk.stride) {
+  for (int tile_pos = 0, tile_id; (tile_id = tile_at(tile_pos)) >= 0; ++tile_pos) {
     const Tile cur = tile_id == seen_id ? seen : sched_tile<C::BM, C::BN>(p, sched, tile_id);
     const int kt_n = __builtin_amdgcn_readfirstlane(slabs_of(cur));
 
@@ -505,6 +553,9 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
       half(1, 0, sn, sbn, 0, READ_NONE, -1);
       wait_vmcnt<WAIT_N>();
       __syncthreads();
+      // queued: this tile's draw, where this wave has no copies in flight (the wait for the counter's answer then
+      // waits for nothing else)
+      if (LAYOUT == LAYOUT_TN && queued && kt == 0 && threadIdx.x == 0) draw_from(tile_pos + 1);
       sc = sc_next;
       half(1, 1, sn, sbn, 0, READ_CATCH_UP, 0);
       ++ring;

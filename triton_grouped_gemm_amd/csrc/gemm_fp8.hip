@@ -79,7 +79,8 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   static_assert(!DEEP || !KGROUP, "the weight-streaming configuration is M-grouped");
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  const auto& sched = *reinterpret_cast<const SchedTableT<kFastMaxGroups>*>(smem + SCHED_AT);
+  auto& sched_rw = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + SCHED_AT);
+  const auto& sched = sched_rw;
   const int64_t num_tiles = sched_num_tiles<C::BM, C::BN>(p, sched);
 
   const uint32_t smem_addr = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
@@ -127,7 +128,14 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
     int s_bytes, kt_n, issued;
     int k_left;  // K-grouped: bytes of the group's token range not yet issued
   };
-  auto slabs_of = [&](const Tile& t) -> int { return KGROUP ? (int)((t.k1 - t.k0 + BKB - 1) / BKB) : (p.K + BKB - 1) / BKB; };
+  // Queued launches (K-grouped, see tile_at below and gemm_fast.hip) give the tiles of an empty group one slab of
+  // nothing instead of none, so that the copy stream advances by exactly one tile per tile.
+  const bool queued = KGROUP && p.queue != nullptr;
+  auto slabs_of = [&](const Tile& t) -> int {
+    if (!KGROUP) return (p.K + BKB - 1) / BKB;
+    const int n = (int)((t.k1 - t.k0 + BKB - 1) / BKB);
+    return queued && n == 0 ? 1 : n;
+  };
   auto make_io = [&](const Tile& t) {
     TileIo io;
     const int64_t k0 = KGROUP ? t.k0 : 0;
@@ -167,46 +175,76 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   // interleaved sweeps); K-grouped: interleaved, since a tile's cost follows its group's token count.
   const TileWalk walk64 = sched_walk(num_tiles, !KGROUP && p.tile_split);
   struct { int first, end, stride; } walk = {(int)walk64.first, (int)walk64.end, (int)walk64.stride};
+  // The workgroup's pos-th tile (-1 past its last one): the static walk, or, queued, ids drawn from the counter in
+  // global memory by thread 0 and passed on through a ring of eight words in the group table's scan scratch: one
+  // draw per tile, on through short tiles up to the first one of kLongTile slabs or kQueueAhead tiles ahead (the
+  // protocol and why it is safe are described in gemm_fast.hip).
+  constexpr int kQueueAhead = 5, kLongTile = 5;
+  int32_t* const qring = reinterpret_cast<int32_t*>(sched_rw.scan_);
+  const int total_tiles = (int)num_tiles;
+  auto tile_at = [&](int pos) -> int {
+    if (queued) {
+      const int id = __builtin_amdgcn_readfirstlane(qring[pos & 7]);
+      return id < total_tiles ? id : -1;
+    }
+    const int64_t id = walk.first + (int64_t)pos * walk.stride;
+    return id < walk.end ? (int)id : -1;
+  };
+  int q_drawn = 0, q_victim = 0;  // thread 0: ids drawn so far, counters found exhausted (see sched_draw_tile)
+  auto draw_from = [&](int from) {
+    for (int j = from; j < from + kQueueAhead; ++j) {
+      if (j >= q_drawn) {
+        qring[j & 7] = sched_draw_tile(p.queue, total_tiles, q_victim);
+        ++q_drawn;
+      }
+      const int id = qring[j & 7];
+      if (id >= total_tiles || slabs_of(sched_tile<C::BM, C::BN>(p, sched, id)) >= kLongTile) break;
+    }
+  };
+  if (queued) {
+    if (threadIdx.x == 0) draw_from(0);
+    __syncthreads();
+  }
   TileIo feed;
-  int feed_id;
+  int feed_pos = 0;
   // The multiplying loop looks every tile up one tile ahead (it needs the tile's weight scales early); the feed
   // reaches that tile later and reuses the lookup instead of repeating its chain of dependent LDS reads.
   Tile nt;
   int nt_id = -1;
   // DEEP: the B copies have a cursor of their own, one slab ahead of `feed` (which then serves A and the scales)
   TileIo feedb;
-  int feedb_id = -1;
-  auto feedb_seek = [&](int id) {
+  int feedb_pos = 0;
+  auto feedb_seek = [&](int pos) {
     feedb.kt_n = 0;
     feedb.issued = 0;
     feedb.a_base = feedb.b_base = feedb.s_base = (uint64_t)p.A;
     feedb.a_left = feedb.b_left = 0;
     feedb.s_bytes = 0;
     feedb.k_left = 0;
-    for (; id < walk.end; id += walk.stride) {
+    for (int id; (id = tile_at(pos)) >= 0; ++pos) {
       const Tile tt = id == nt_id ? nt : sched_tile<C::BM, C::BN>(p, sched, id);
       if (slabs_of(tt) > 0) {
         feedb = make_io(tt);
         break;
       }
     }
-    feedb_id = id;
+    feedb_pos = pos;
   };
-  auto feed_seek = [&](int id) {
+  auto feed_seek = [&](int pos) {
     feed.kt_n = 0;
     feed.issued = 0;
     feed.a_base = feed.b_base = feed.s_base = (uint64_t)p.A;
     feed.a_left = feed.b_left = 0;
     feed.s_bytes = 0;
     feed.k_left = 0;
-    for (; id < walk.end; id += walk.stride) {
+    for (int id; (id = tile_at(pos)) >= 0; ++pos) {
       const Tile tt = id == nt_id ? nt : sched_tile<C::BM, C::BN>(p, sched, id);
       if (slabs_of(tt) > 0) {
         feed = make_io(tt);
         break;
       }
     }
-    feed_id = id;
+    feed_pos = pos;
   };
   struct SlabCopy {
     i32x4_t ra, rb, rs;
@@ -223,7 +261,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
     feedb.b_base += BKB;
     feedb.b_left -= BKB;
     feedb.issued += 1;
-    if (live && feedb.issued >= feedb.kt_n) feedb_seek(feedb_id + walk.stride);
+    if (live && feedb.issued >= feedb.kt_n) feedb_seek(feedb_pos + 1);
   };
   auto begin_slab = [&](int buf, int buf_b = 0) {
     SlabCopy sc;
@@ -246,7 +284,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
     feed.b_left -= BKB;
     feed.s_base += (uint64_t)p.m_total * 4;
     feed.issued += 1;
-    if (live && feed.issued >= feed.kt_n) feed_seek(feed_id + walk.stride);
+    if (live && feed.issued >= feed.kt_n) feed_seek(feed_pos + 1);
     if (DEEP) begin_b(sc, buf_b);
     return sc;
   };
@@ -281,8 +319,8 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   // DEEP: per slab the scale, A and then B copies go out, the B copies for a slab one further ahead; the wait lets
   // the CB most recent copies -- those B copies -- stay in flight (loads complete in order).
   constexpr int WAIT_N = DEEP ? CB : 0;
-  if (DEEP) feedb_seek(walk.first);
-  feed_seek(walk.first);
+  if (DEEP) feedb_seek(0);
+  feed_seek(0);
   {
     SlabCopy s0 = begin_slab(0, 0);
 #pragma unroll
@@ -314,8 +352,9 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   int ring3 = 0;  // ring % 3 (DEEP: the B buffer of the current slab)
 
   float sbv_next = 0.f;
-  if (walk.first < walk.end) {
-    nt = sched_tile<C::BM, C::BN>(p, sched, walk.first);
+  if (tile_at(0) >= 0) {
+    nt = sched_tile<C::BM, C::BN>(p, sched, tile_at(0));
+    nt_id = tile_at(0);
     load_sbv(nt, sbv_next);
     if (DEEP && BLOCK) wait_vmcnt<0>();  // there the load is not the compiler's to wait for, and the first slab reads it
   }
@@ -334,13 +373,14 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
       for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
   };
 
-  for (int tile_id = walk.first; tile_id < walk.end; tile_id += walk.stride) {
-    const Tile cur = nt;
+  for (int tile_pos = 0, tile_id; (tile_id = tile_at(tile_pos)) >= 0; ++tile_pos) {
+    const Tile cur = (!queued || tile_id == nt_id) ? nt : sched_tile<C::BM, C::BN>(p, sched, tile_id);
     const int kt_n = __builtin_amdgcn_readfirstlane(slabs_of(cur));
     float sbv = sbv_next;
-    if (tile_id + walk.stride < walk.end) {
-      nt = sched_tile<C::BM, C::BN>(p, sched, tile_id + walk.stride);
-      nt_id = tile_id + walk.stride;
+    // (queued launches look nothing up ahead here: the next id may not be drawn yet, and they need no weight scales)
+    if (const int next_id = queued ? -1 : tile_at(tile_pos + 1); next_id >= 0) {
+      nt = sched_tile<C::BM, C::BN>(p, sched, next_id);
+      nt_id = next_id;
       load_sbv(nt, sbv_next);
     }
 
@@ -406,6 +446,8 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
           wait_vmcnt_lgkmcnt0<WAIT_N>();
           if (BLOCK) asm volatile("" : "+v"(sbv_next));  // everything older than the newest B copies has landed: touching it costs no wait
           __syncthreads();
+          // queued: this tile's draw, where this wave has nothing in flight
+          if (KGROUP && queued && kt == 0 && threadIdx.x == 0) draw_from(tile_pos + 1);
           sc = scn;
           fa[0] = load_frag(sn + wm0 * 128);
         }

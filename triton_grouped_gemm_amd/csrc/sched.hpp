@@ -366,4 +366,29 @@ TGG_DEV TileWalk sched_walk(int64_t num_tiles, bool split) {
   return sched_walk_of(num_tiles, split, (int)gridDim.x, (int)blockIdx.x);
 }
 
+// Work queue of the K-grouped tuned kernels: eight counters in global memory, one per XCD (zero at launch).  The
+// tile space is cut into runs of R neighbouring tiles (R = workgroups per XCD; neighbours are tiles of one group,
+// which share operand panels in an XCD's L2), and the runs are dealt to the XCDs in order of decreasing cost, back
+// and forth (0..7, 7..0, ...) so that no XCD always gets the dearest of eight.  Within an XCD a tile goes to
+// whichever workgroup asks next: like the static interleaved walk the XCD works through runs of neighbours, but a
+// workgroup that drew expensive tiles draws fewer.  A workgroup whose own XCD has nothing left takes from the
+// next XCD's counter, and so on round the ring: what the deal leaves uneven is evened out at the end.  For every
+// counter the ids grow with the number of draws, so one id at or beyond `total` means that counter is exhausted.
+// `victim` (0 at first; kept by the drawing thread) counts the counters found exhausted so far; returns an id at
+// or beyond `total` when all eight are.
+TGG_DEV int sched_draw_tile(int32_t* queue, int total, int& victim) {
+  const int P = (int)gridDim.x;
+  if ((P & 7) != 0) return atomicAdd(queue, 1);
+  const int x = (int)blockIdx.x & 7, R = P >> 3;
+  while (victim < 8) {
+    const int xq = (x + victim) & 7;
+    const int n = atomicAdd(queue + xq, 1);
+    const int run = n / R;
+    const int id = (run * 8 + ((run & 1) ? 7 - xq : xq)) * R + n % R;
+    if (id < total) return id;
+    ++victim;
+  }
+  return total;
+}
+
 }  // namespace tgg

@@ -58,7 +58,9 @@ def k_grouped_gemm(A: Tensor, B: Tensor, size_per_group: Tensor, group_start: Op
         group_start = group_end - size_per_group
     group_start = group_start.to(device=A.device, dtype=torch.int32).contiguous()
     group_end = group_end.to(device=A.device, dtype=torch.int32).contiguous()
-    _native.call("tgg_k_grouped_gemm", A.data_ptr(), B.data_ptr(), C.data_ptr(), group_start.data_ptr(),
+    # tile-id counter of the kernel's work queue (a tile costs what its group has tokens; see include/tgg_amd.h)
+    queue = torch.zeros(_native.QUEUE_WORDS, dtype=torch.int32, device=A.device)
+    _native.call("tgg_k_grouped_gemm_queued", A.data_ptr(), B.data_ptr(), C.data_ptr(), group_start.data_ptr(),
                  group_end.data_ptr(), num_groups, M_DIM, N_DIM, K_TOTAL, _dtype_code(A.dtype), int(numSM),
-                 _native.stream_of(A))
+                 queue.data_ptr(), _native.stream_of(A))
     return C

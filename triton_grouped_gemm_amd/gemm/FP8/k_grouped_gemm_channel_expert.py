@@ -41,7 +41,10 @@ def matmul(x_fp8: Tensor, x_scale: Tensor, y_fp8: Tensor, y_scale: Tensor, token
     ys = _expert_major(y_scale, N, num_groups)
     tokens = tokens_per_expert.to(device=x_fp8.device, dtype=torch.int32).contiguous()
     output = torch.empty((num_groups, M, N), dtype=torch.bfloat16, device=x_fp8.device)
-    _native.call("tgg_k_grouped_gemm_fp8_channel", x_fp8.data_ptr(), xs.data_ptr(), y_fp8.data_ptr(), ys.data_ptr(),
-                 output.data_ptr(), tokens.data_ptr(), num_groups, M, N, K, _FMT.get(int(dtype_a), _native.E5M2),
-                 _FMT.get(int(dtype_b), _native.E5M2), -1, _native.stream_of(x_fp8))
+    # tile-id counter of the kernel's work queue (a tile costs what its group has tokens; see include/tgg_amd.h)
+    queue = torch.zeros(_native.QUEUE_WORDS, dtype=torch.int32, device=x_fp8.device)
+    _native.call("tgg_k_grouped_gemm_fp8_channel_queued", x_fp8.data_ptr(), xs.data_ptr(), y_fp8.data_ptr(),
+                 ys.data_ptr(), output.data_ptr(), tokens.data_ptr(), num_groups, M, N, K,
+                 _FMT.get(int(dtype_a), _native.E5M2), _FMT.get(int(dtype_b), _native.E5M2), -1, queue.data_ptr(),
+                 _native.stream_of(x_fp8))
     return output
