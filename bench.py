@@ -32,16 +32,16 @@ PEAK_HBM_GBS = 8000.0
 # plain 1 GiB device copy: x2.0 and x1.0).  The runs and their figures are listed in profiles/hbm_traffic.txt.
 # FETCH_SIZE includes L2 fills served by the memory-side cache, so these are upper bounds on DRAM traffic.
 MEASURED_TRAFFIC_GB = {
-    "bf16_m_grouped_gateup_nt": 12.18,
-    "bf16_m_grouped_gateup_nn": 11.95,
-    "bf16_m_grouped_gateup_fp8_out": 10.47,
-    "bf16_m_grouped_down_nt": 5.42,
-    "bf16_m_grouped_down_nn": 5.37,
-    "bf16_masked_decode": 2.54,
-    "bf16_k_grouped_wgrad": 29.13,
-    "fp8_block_m_grouped": 27.24,
-    "fp8_channel_m_grouped": 28.31,
-    "fp8_channel_k_grouped": 17.92,
+    "bf16_m_grouped_gateup_nt": 11.98,
+    "bf16_m_grouped_gateup_nn": 11.94,
+    "bf16_m_grouped_gateup_fp8_out": 10.69,
+    "bf16_m_grouped_down_nt": 5.38,
+    "bf16_m_grouped_down_nn": 5.42,
+    "bf16_masked_decode": 2.51,
+    "bf16_k_grouped_wgrad": 28.31,
+    "fp8_block_m_grouped": 29.07,
+    "fp8_channel_m_grouped": 27.73,
+    "fp8_channel_k_grouped": 18.05,
     "quant_trans128": 8.12,
     "moe_permute": 3.06,      # the row mover (the sort kernels move < 1 % of that)
     "moe_unpermute": 3.07,
