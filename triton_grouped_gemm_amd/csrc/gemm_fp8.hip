@@ -213,6 +213,8 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   int nt_id = -1;
   // DEEP: the B copies have a cursor of their own, one slab ahead of `feed` (which then serves A and the scales)
   TileIo feedb;
+  Tile seen;          // queued launches: the tile the feed looked up last
+  int seen_id = -1;
   int feedb_pos = 0;
   auto feedb_seek = [&](int pos) {
     feedb.kt_n = 0;
@@ -239,6 +241,10 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
     feed.k_left = 0;
     for (int id; (id = tile_at(pos)) >= 0; ++pos) {
       const Tile tt = id == nt_id ? nt : sched_tile<C::BM, C::BN>(p, sched, id);
+      if (queued) {  // no look-ahead by the multiplying loop there: it reuses this lookup instead
+        seen = tt;
+        seen_id = id;
+      }
       if (slabs_of(tt) > 0) {
         feed = make_io(tt);
         break;
@@ -374,7 +380,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   };
 
   for (int tile_pos = 0, tile_id; (tile_id = tile_at(tile_pos)) >= 0; ++tile_pos) {
-    const Tile cur = (!queued || tile_id == nt_id) ? nt : sched_tile<C::BM, C::BN>(p, sched, tile_id);
+    const Tile cur = (!queued || tile_id == nt_id) ? nt : (tile_id == seen_id ? seen : sched_tile<C::BM, C::BN>(p, sched, tile_id));
     const int kt_n = __builtin_amdgcn_readfirstlane(slabs_of(cur));
     float sbv = sbv_next;
     // (queued launches look nothing up ahead here: the next id may not be drawn yet, and they need no weight scales)
