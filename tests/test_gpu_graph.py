@@ -144,3 +144,23 @@ def test_deep_gemm_shaped_wrappers_can_be_captured(dev):
         torch.cuda.synchronize()
         assert torch.equal(out16, ref16), f"replay {it}"
         assert torch.equal(out8, ref8), f"replay {it} (fp8)"
+
+
+def test_k_grouped_wrapper_with_its_work_queue_can_be_captured(dev):
+    """k_grouped_gemm clears the kernel's tile counters with a small fill kernel on every call; captured, that fill is
+    part of the graph, so every replay starts from zero counters.  Replays with other token counts (read on the
+    device) must equal the eager call."""
+    G, Kt, Mdim, N = 6, 3072, 264, 520
+    a, b = _randn((Kt, Mdim), 41, dev), _randn((Kt, N), 42, dev)
+    sizes = torch.tensor([512] * G, dtype=torch.int32, device=dev)
+    k_grouped_gemm(a, b, sizes)  # first launch outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = k_grouped_gemm(a, b, sizes)
+    for it, routing in enumerate([[512] * G, [3000, 0, 0, 8, 0, 64], [0, 1024, 1024, 0, 1000, 24], [512] * G]):
+        sizes.copy_(torch.tensor(routing, dtype=torch.int32))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, k_grouped_gemm(a, b, sizes)), f"replay {it}"
