@@ -247,8 +247,8 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
   // ring of eight words in the group table's scan scratch; readers use plain LDS reads, so an id must be drawn a
   // workgroup barrier before anyone can ask for it.  Who asks first is the copy stream: it runs two slabs ahead of
   // the multiplies and looks the next tile up as soon as it has requested a tile's last slab.  Thread 0 draws once
-  // per tile, right after the barrier of the tile's first slab (what it writes there is seen by all from the
-  // second slab after that one on), and draws on through short tiles until it has drawn one of at least
+  // per tile, right before the barrier of the tile's first slab (what it writes there is seen by all from the
+  // next slab on at the latest), and draws on through short tiles until it has drawn one of at least
   // kLongTile slabs -- that one gives the next draw time enough -- or is kQueueAhead tiles ahead (enough for any
   // run of one-slab tiles).  So a workgroup commits itself to one expensive tile beyond the one in work, not more:
   // committing to several is what spoils the balance when a workgroup has only a dozen tiles in all.  Ids at or
@@ -552,10 +552,11 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
       half(0, 1, sa, sba, 1, READ_ROLL, -1, true);
       half(1, 0, sn, sbn, 0, READ_NONE, -1);
       wait_vmcnt<WAIT_N>();
-      __syncthreads();
       // queued: this tile's draw, where this wave has no copies in flight (the wait for the counter's answer then
-      // waits for nothing else)
+      // waits for nothing else) and in front of the barrier: wave 0 is the first-served wave of its SIMD and tends
+      // to reach the barrier early, so part of the answer's latency falls into time it would spend waiting there
       if (LAYOUT == LAYOUT_TN && queued && kt == 0 && threadIdx.x == 0) draw_from(tile_pos + 1);
+      __syncthreads();
       sc = sc_next;
       half(1, 1, sn, sbn, 0, READ_CATCH_UP, 0);
       ++ring;

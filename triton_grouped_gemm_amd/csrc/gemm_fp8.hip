@@ -451,9 +451,9 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
           // fragment was requested a row block ago) are complete: after the barrier the buffer is overwritten
           wait_vmcnt_lgkmcnt0<WAIT_N>();
           if (BLOCK) asm volatile("" : "+v"(sbv_next));  // everything older than the newest B copies has landed: touching it costs no wait
-          __syncthreads();
-          // queued: this tile's draw, where this wave has nothing in flight
+          // queued: this tile's draw, where this wave has nothing in flight, in front of the barrier (gemm_fast.hip)
           if (KGROUP && queued && kt == 0 && threadIdx.x == 0) draw_from(tile_pos + 1);
+          __syncthreads();
           sc = scn;
           fa[0] = load_frag(sn + wm0 * 128);
         }
