@@ -187,7 +187,8 @@ int tgg_moe_unpermute_bwd(const void* grad_output, const void* fwd_input, const 
  * what the reference's grouped_launch / m_indices_pad tile enumeration guarantees
  * (gemm/BF16/m_grouped_gemm_TMA.py:55-71, :297-326): every tile of the padded tile space exactly once.
  *   sizes  host array [G]; mode 0 M-grouped, 1 rows padded to `aux`, 2 masked with `aux` rows per group,
- *          4 K-grouped by token counts (`aux` = total tokens, m_total = rows of each output)
+ *          4 K-grouped by token counts (`aux` = total tokens, m_total = rows of each output; the tile space lists
+ *          the groups by decreasing token count, and what is reported is the fixed walk, not a queued launch's draws)
  *   tile   256 (tuned kernels) or 128 (shape-agnostic kernel); split as in the "tile_split" option
  *   out    [capacity][6] = workgroup, position in its walk, group, first row, valid rows, first column */
 int tgg_debug_tile_order(const int64_t* sizes, int G, int mode, int64_t m_total, int64_t aux, int N, int tile,
