@@ -60,6 +60,20 @@ WORKLOADS = {
     "fp8_block_m_grouped": ("fp8", 3072, 4096, True),
     "fp8_channel_m_grouped": ("fp8c", 3072, 4096, True),     # per-token x per-channel scales, same shape
     "fp8_channel_k_grouped": ("fp8ck", 4096, 3072, False),   # N_DIM, M_DIM; tokens along K
+    # The other shapes of the reference's published tables (README.md:99-140: 16 M-grouped and 8 K-grouped cases on
+    # 128 uniform groups of 5120 rows -- run these with --uniform-groups to sit beside them) ...
+    "bf16_m_grouped_235b_gateup_nt": ("mg", 3072, 4096, True),
+    "bf16_m_grouped_235b_gateup_nn": ("mg", 3072, 4096, False),
+    "bf16_m_grouped_235b_down_nt": ("mg", 4096, 1536, True),
+    "bf16_m_grouped_235b_down_nn": ("mg", 4096, 1536, False),
+    "bf16_k_grouped_30b_gateup": ("kg", 2048, 1536, False),
+    "bf16_k_grouped_30b_down": ("kg", 768, 2048, False),
+    "bf16_k_grouped_235b_down": ("kg", 1536, 4096, False),
+    # ... and its two FP8 examples (README.md:168-169; gemm/FP8/m_grouped_gemm_channel_expert.py:293-308,
+    # gemm/FP8/k_grouped_gemm_channel_expert.py:276-296): 32 experts with fixed token counts, activations e5m2,
+    # weights e4m3fn; the K-grouped one with every expert's tokens padded to a multiple of 128.
+    "fp8_channel_m_grouped_readme": ("fp8c", 6144, 5120, True, dict(sizes=[509, 3587, 125, 3971] * 8, fmt_a="e5m2")),
+    "fp8_channel_k_grouped_readme": ("fp8ck", 6144, 5120, False, dict(sizes=[512, 3584, 128, 3968] * 8, fmt_a="e5m2")),
     "quant_trans128": ("quant", 4096, 0, False),
     # MoE token movement either side of the GEMMs: 81920 tokens x top-8 = 655360 rows of 2048 bf16
     "moe_permute": ("permute", 2048, 8, False),       # hidden, topK
@@ -94,12 +108,19 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
     build_workload.operands = {}
     from triton_grouped_gemm_amd import workloads as wl
     from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm_TMA import m_grouped_gemm
-    kind, N, K, trans_b = WORKLOADS[name]
+    kind, N, K, trans_b, *extra = WORKLOADS[name]
+    opts = extra[0] if extra else {}
     G = groups or globals()["G"]
     M_TOTAL = m_total or globals()["M_TOTAL"]
-    sizes_cpu = wl.uniform_sizes(G, M_TOTAL) if uniform else wl.dirichlet_multinomial_sizes(G, M_TOTAL, 128, seed=seed)
+    if "sizes" in opts and not groups:  # the workload states its own group sizes
+        sizes_cpu = torch.tensor(opts["sizes"], dtype=torch.int32)
+        G, M_TOTAL = len(opts["sizes"]), int(sum(opts["sizes"]))
+        size_tag = "as the reference's example: " + " ".join(map(str, opts["sizes"][:4])) + f" x {G // 4}"
+    else:
+        sizes_cpu = wl.uniform_sizes(G, M_TOTAL) if uniform else wl.dirichlet_multinomial_sizes(G, M_TOTAL, 128, seed=seed)
+        size_tag = f"uniform, {M_TOTAL // G} rows per group" if uniform else "dirichlet-multinomial, 128-aligned"
     sizes = sizes_cpu.to(dev)
-    size_tag = f"uniform, {M_TOTAL // G} rows per group" if uniform else "dirichlet-multinomial, 128-aligned"
+    fp8_a = torch.float8_e5m2 if opts.get("fmt_a") == "e5m2" else torch.float8_e4m3fn
     bounds = [(int(s0), int(s0 + n)) for s0, n in zip((sizes_cpu.cumsum(0) - sizes_cpu).tolist(), sizes_cpu.tolist())]
     if kind == "mg":
         a = wl.randn_bf16((M_TOTAL, K), K ** -0.5, seed + 1, dev)
@@ -210,7 +231,7 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
     if kind == "fp8c":
         from triton_grouped_gemm_amd.gemm.FP8.m_grouped_gemm_channel_expert import gmm_fp8_act_per_channel_w_per_expert
         gen = torch.Generator(device=dev).manual_seed(seed + 3)
-        a = wl.randn_bf16((M_TOTAL, K), 1.0, seed + 1, dev).to(torch.float8_e4m3fn)
+        a = wl.randn_bf16((M_TOTAL, K), 1.0, seed + 1, dev).to(fp8_a)
         w = wl.randn_bf16((G, N, K), 1.0, seed + 2, dev).to(torch.float8_e4m3fn)
         sa = torch.rand(M_TOTAL, 1, device=dev, generator=gen) + 0.5
         sb = torch.rand(G * N, device=dev, generator=gen) + 0.5
@@ -228,21 +249,24 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
         build_workload.vendor_out = c_ref
         build_workload.vendor_kind = "torch._scaled_mm per group (hipBLASLt), row-wise scales, same operands"
         return (fn, 2.0 * M_TOTAL * N * K, nbytes, "fp8",
-                dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, recipe="per-token x per-channel scales, e4m3fn",
+                dict(workload=name, G=G, M=M_TOTAL, N=N, K=K,
+                     recipe="per-token x per-channel scales, " + ("e5m2 x e4m3fn" if fp8_a == torch.float8_e5m2 else "e4m3fn"),
                      group_sizes=size_tag, seed=seed), None)
     if kind == "fp8ck":
         from triton_grouped_gemm_amd.gemm.FP8.k_grouped_gemm_channel_expert import matmul as k_grouped_fp8
         m_dim, n_dim = K, N
         gen = torch.Generator(device=dev).manual_seed(seed + 3)
-        x = wl.randn_bf16((m_dim, M_TOTAL), 1.0, seed + 1, dev).to(torch.float8_e4m3fn)
+        x = wl.randn_bf16((m_dim, M_TOTAL), 1.0, seed + 1, dev).to(fp8_a)
         y = wl.randn_bf16((n_dim, M_TOTAL), 1.0, seed + 2, dev).to(torch.float8_e4m3fn)
         xs = torch.rand(m_dim, G, device=dev, generator=gen) + 0.5
         ys = torch.rand(n_dim, G, device=dev, generator=gen) + 0.5
-        fn = lambda: k_grouped_fp8(x, xs, y, ys, sizes, m_dim, n_dim, M_TOTAL, G)
+        code_a = 2 if fp8_a == torch.float8_e5m2 else 1
+        fn = lambda: k_grouped_fp8(x, xs, y, ys, sizes, m_dim, n_dim, M_TOTAL, G, dtype_a=code_a, dtype_b=1)
         nbytes = 1.0 * M_TOTAL * (m_dim + n_dim) + 4.0 * G * (m_dim + n_dim) + 2.0 * G * m_dim * n_dim
         return (fn, 2.0 * M_TOTAL * m_dim * n_dim, nbytes, "fp8",
-                dict(workload=name, G=G, M=m_dim, N=n_dim, K_total=M_TOTAL, recipe="per-channel x per-expert scales, e4m3fn",
-                     seed=seed), None)
+                dict(workload=name, G=G, M=m_dim, N=n_dim, K_total=M_TOTAL,
+                     recipe="per-channel x per-expert scales, " + ("e5m2 x e4m3fn" if code_a == 2 else "e4m3fn"),
+                     group_sizes=size_tag, seed=seed), None)
     if kind == "quant":
         from triton_grouped_gemm_amd.quant.trans_per_block_quant_expand_128x import trans_per_block_quant_expand_128x
         x = wl.randn_bf16((M_TOTAL, N), 1.0, seed + 1, dev)
@@ -396,7 +420,7 @@ def main() -> int:
                             sample=sample, host_cpus=os.cpu_count())
 
     line = {
-        "metric": METRICS[kind], "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps,
+        "metric": METRICS[kind].replace("G=128", f"G={config['G']}") if "G" in config else METRICS[kind], "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dtype_tag, "data": "synthetic-zeros" if args.zeros else "synthetic", "config": config,
         "roofline": roofline, "cpu_baseline": cpu_baseline, "vendor_loop": vendor,
