@@ -370,7 +370,8 @@ def test_many_groups_exact(dev, variant, G):
     [0, 0, 0, 9000],                                          # empty groups first in index order
     [(53 * g * g + 17 * g) % 3000 for g in range(96)],
 ])
-def test_k_grouped_work_queue_equals_fixed_assignment(dev, sizes):
+@pytest.mark.parametrize("num_cu", [-1, 100, 64, 8])  # 100: not a multiple of 8, one counter; 8: one workgroup per XCD
+def test_k_grouped_work_queue_equals_fixed_assignment(dev, sizes, num_cu):
     """tgg_k_grouped_gemm_queued (tile ids drawn from counters in device memory, largest groups first) against
     tgg_k_grouped_gemm (fixed assignment) and the oracle: same bits, whichever workgroup computes a tile; the
     counters end at the number of draws, at least one per tile."""
@@ -386,9 +387,9 @@ def test_k_grouped_work_queue_equals_fixed_assignment(dev, sizes):
     queue = torch.zeros(_native.QUEUE_WORDS, dtype=torch.int32, device=dev)
     st = _native.stream_of(a)
     _native.call("tgg_k_grouped_gemm", a.data_ptr(), b.data_ptr(), fixed.data_ptr(), start.data_ptr(), end.data_ptr(),
-                 G, Mdim, N, Kt, _native.BF16, -1, st)
+                 G, Mdim, N, Kt, _native.BF16, num_cu, st)
     _native.call("tgg_k_grouped_gemm_queued", a.data_ptr(), b.data_ptr(), drawn.data_ptr(), start.data_ptr(),
-                 end.data_ptr(), G, Mdim, N, Kt, _native.BF16, -1, queue.data_ptr(), st)
+                 end.data_ptr(), G, Mdim, N, Kt, _native.BF16, num_cu, queue.data_ptr(), st)
     assert torch.equal(fixed, drawn)
     tiles = G * ((Mdim + 255) // 256) * ((N + 255) // 256)
     assert int(queue.sum()) >= tiles
