@@ -202,6 +202,13 @@ int tgg_debug_tile_order(const int64_t* sizes, int G, int mode, int64_t m_total,
 int tgg_debug_row_tiles(const int64_t* sizes, int G, int mode, int64_t m_total, int64_t aux, int tile, int n_chunk,
                         int64_t* out, int64_t capacity, int64_t* num_row_tiles);
 
+/* Test hook, host only: the deal of the K-grouped kernels' work queue.  out[xq][n] (row-major, [8][draws]) = the tile
+ * id behind the n-th draw from XCD xq's counter on a grid of `grid` workgroups (a multiple of 8; other grids use
+ * one counter whose draws are the ids themselves).  The reference has no counterpart (its K-grouped kernels walk
+ * tiles at a fixed stride, gemm/BF16/k_grouped_gemm_TMA.py:124-135); what must hold is that the eight sequences
+ * together list every id once and each of them in growing order. */
+int tgg_debug_queue_order(int grid, int draws, int32_t* out);
+
 /* Library controls (process-wide, meant for tests and tuning; returns 1 for an unknown key):
  *   "force_generic" 0/1  route every GEMM through the shape-agnostic kernel
  *   "variant"       int  tile configuration of the tuned kernels (16-bit, and FP8 M-grouped): 0 (default) = chosen per launch on the

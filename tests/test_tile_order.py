@@ -165,3 +165,28 @@ def test_row_tile_lookup_padded_and_masked():
     assert row_tiles(sizes, MG_PAD, 512, 128, 128) == [[0, 0, 100], [2, 128, 128], [2, 256, 2], [3, 384, 128]]
     assert row_tiles([512, 0, 77, 300], MASKED, 2048, 512, 256) == [
         [0, 0, 256], [0, 256, 256], [2, 1024, 77], [3, 1536, 256], [3, 1792, 44]]
+
+
+@pytest.mark.parametrize("grid", [8, 64, 104, 256])
+def test_work_queue_deals_every_tile_once_and_each_counter_in_growing_order(grid):
+    """The K-grouped kernels draw tile ids from eight counters (one per XCD).  A counter is taken for exhausted at
+    its first id beyond the tile space, and workgroups then steal from the other counters: that is only right if
+    each counter's ids grow with the number of draws and the eight sequences together are a permutation of the ids.
+    The deal hands out runs of grid/8 neighbouring tiles, eight runs per pass, forwards and backwards in turn."""
+    lib = _native.load()
+    R, draws = grid // 8, 7 * (grid // 8) + 3
+    out = np.full((8, draws), -1, dtype=np.int32)
+    assert lib.tgg_debug_queue_order(grid, draws, out.ctypes.data) == 0, _native.last_error()
+    assert (np.diff(out, axis=1) > 0).all()
+    full = 7 * grid  # the first seven passes are dealt completely
+    ids = np.sort(out[out < full])
+    assert np.array_equal(ids, np.arange(full))
+    runs = out[:, :7 * R].reshape(8, 7, R)
+    assert (np.diff(runs, axis=2) == 1).all(), "a run is R neighbouring tiles"
+    first = runs[:, :, 0] // R  # run number in the tile space, by counter and pass
+    for k in range(7):
+        order = np.argsort(first[:, k])
+        assert np.array_equal(first[order, k], 8 * k + np.arange(8))
+        assert np.array_equal(order, np.arange(8) if k % 2 == 0 else np.arange(8)[::-1]), "back and forth"
+    bad = np.zeros((8, 4), dtype=np.int32)
+    assert lib.tgg_debug_queue_order(100, 4, bad.ctypes.data) == 1  # not a multiple of 8: one counter, ids in order

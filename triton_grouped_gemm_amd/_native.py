@@ -45,6 +45,7 @@ SIGNATURES = {
     "tgg_moe_unpermute_bwd": [_P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _P],
     "tgg_debug_tile_order": [_P, _I, _I, _L, _L, _I, _I, _I, _I, _P, _L, _P],
     "tgg_debug_row_tiles": [_P, _I, _I, _L, _L, _I, _I, _P, _L, _P],
+    "tgg_debug_queue_order": [_I, _I, _P],
     "tgg_set_option": [c_char_p, _I],
     "tgg_version": [],
 }

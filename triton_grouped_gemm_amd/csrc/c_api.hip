@@ -471,6 +471,15 @@ int tgg_debug_tile_order(const int64_t* sizes, int G, int mode, int64_t m_total,
   return set_error("tile must be 256 (tuned kernels) or 128 (shape-agnostic kernel)");
 }
 
+int tgg_debug_queue_order(int grid, int draws, int32_t* out) {
+  if (!out) return set_error("null pointer");
+  if (grid < 8 || (grid & 7) != 0) return set_error("a grid of %d workgroups draws from one counter: ids in order", grid);
+  if (draws < 0) return set_error("negative number of draws");
+  for (int xq = 0; xq < 8; ++xq)
+    for (int n = 0; n < draws; ++n) out[(int64_t)xq * draws + n] = sched_queue_id(n, xq, grid >> 3);
+  return 0;
+}
+
 int tgg_debug_row_tiles(const int64_t* sizes, int G, int mode, int64_t m_total, int64_t aux, int tile, int n_chunk,
                         int64_t* out, int64_t capacity, int64_t* num_row_tiles) {
   if (!sizes || !out || !num_row_tiles) return set_error("null pointer");

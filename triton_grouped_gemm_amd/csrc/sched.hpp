@@ -366,6 +366,13 @@ TGG_DEV TileWalk sched_walk(int64_t num_tiles, bool split) {
   return sched_walk_of(num_tiles, split, (int)gridDim.x, (int)blockIdx.x);
 }
 
+// The tile id behind the n-th draw from XCD xq's counter (R = workgroups per XCD): run n / R of that XCD, which is run
+// xq of the deal's pass n / R when the pass runs forwards (even) and run 7 - xq when it runs backwards.
+TGG_HD int sched_queue_id(int n, int xq, int R) {
+  const int pass = n / R;
+  return (pass * 8 + ((pass & 1) ? 7 - xq : xq)) * R + n % R;
+}
+
 // Work queue of the K-grouped tuned kernels: eight counters in global memory, one per XCD (zero at launch).  The
 // tile space is cut into runs of R neighbouring tiles (R = workgroups per XCD; neighbours are tiles of one group,
 // which share operand panels in an XCD's L2), and the runs are dealt to the XCDs in order of decreasing cost, back
@@ -382,9 +389,7 @@ TGG_DEV int sched_draw_tile(int32_t* queue, int total, int& victim) {
   const int x = (int)blockIdx.x & 7, R = P >> 3;
   while (victim < 8) {
     const int xq = (x + victim) & 7;
-    const int n = atomicAdd(queue + xq, 1);
-    const int run = n / R;
-    const int id = (run * 8 + ((run & 1) ? 7 - xq : xq)) * R + n % R;
+    const int id = sched_queue_id(atomicAdd(queue + xq, 1), xq, R);
     if (id < total) return id;
     ++victim;
   }
