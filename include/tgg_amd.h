@@ -41,7 +41,8 @@ int tgg_m_grouped_gemm_padded(const void* A, const void* B, void* C, const void*
                               int64_t M, int N, int K, int align, int dtype, int num_cu, void* stream);
 
 /* As tgg_m_grouped_gemm_padded, but group g's rows are [row_start[g], row_start[g] + sizes[g]): the groups'
- * regions may lie in any order (they must not overlap; a group has one region).  What a per-row grouped_layout
+ * regions may lie in any order (they must not overlap; a group has one region -- a caller whose expert owns several
+ * passes one group per region, with B holding that expert's weights once per region).  What a per-row grouped_layout
  * that lists experts out of ascending order describes; the reference forwards any such layout to its backend
  * (gemm/deep_gemm_ops.py:24-57). */
 int tgg_m_grouped_gemm_placed(const void* A, const void* B, void* C, const void* sizes, int sizes_i64,

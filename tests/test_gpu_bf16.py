@@ -239,6 +239,26 @@ def test_contiguous_bf16_per_row_layout_in_any_expert_order(dev, variant, layout
     assert bool((out[~valid] == 3.0).all()), "padding rows were written"
 
 
+def test_contiguous_bf16_per_row_layout_with_experts_in_several_regions(dev, variant):
+    """A per-row layout in which two experts own two separate regions each (whole 128-row blocks first, the rest
+    later): every row still gets its own expert's weights, out[r] = a[r] . b[layout[r]]^T, integer inputs, bit
+    for bit; the padded total is the one the reference's check expects (gemm/deep_gemm_ops.py:49-51)."""
+    sizes = [300, 128, 0, 200]
+    lay = [3] * 128 + [0] * 256 + [1] * 128 + [3] * 72 + [-1] * 56 + [0] * 44 + [-1] * 84
+    lay = torch.tensor(lay, dtype=torch.int32)
+    Mp, N, K = lay.numel(), 264, 136
+    a = _ints((Mp, K), 33)
+    b = _ints((len(sizes), N, K), 34)
+    out = torch.full((Mp, N), 3.0, dtype=torch.bfloat16, device=dev)
+    m_grouped_bf16_nt_contiguous(a.to(dev), b.to(dev), torch.tensor(sizes, dtype=torch.int32, device=dev), out=out,
+                                 grouped_layout=lay.to(dev))
+    out = out.cpu()
+    valid = lay >= 0
+    ref = torch.einsum("rk,rnk->rn", a[valid].float(), b[lay[valid].long()].float()).to(torch.bfloat16)
+    assert torch.equal(out[valid], ref)
+    assert bool((out[~valid] == 3.0).all()), "padding rows were written"
+
+
 @pytest.mark.parametrize("trans_b", [True, False])
 def test_masked_small(dev, variant, trans_b):
     G, m_max, N, K = 6, 256, 264, 192

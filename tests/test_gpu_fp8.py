@@ -331,6 +331,31 @@ def test_fp8_block_scaled_per_row_layout_in_any_expert_order(dev, variant):
     assert bool((out[~valid] == 9.0).all()), "padding rows were written"
 
 
+def test_fp8_block_scaled_per_row_layout_with_experts_in_several_regions(dev, variant):
+    """Two experts own two separate regions each: every row gets its own expert's weights and weight scales
+    (small-integer codes and power-of-two scales: the closed form is exact)."""
+    g = torch.Generator().manual_seed(72)
+    sizes, K, N = [300, 128, 0, 200], 384, 256
+    lay = torch.tensor([3] * 128 + [0] * 256 + [1] * 128 + [3] * 72 + [-1] * 56 + [0] * 44 + [-1] * 84, dtype=torch.int32)
+    Mp, G, kb = lay.numel(), len(sizes), K // 128
+    aq = torch.randint(-3, 4, (Mp, K), generator=g).float()
+    bq = torch.randint(-3, 4, (G, N, K), generator=g).float()
+    pw = torch.tensor([0.25, 0.5, 1.0, 2.0])
+    sa = pw[torch.randint(0, 4, (Mp, kb), generator=g)]
+    sb = pw[torch.randint(0, 4, (G, N // 128, kb), generator=g)]
+    out = torch.full((Mp, N), 9.0, dtype=torch.bfloat16, device=dev)
+    m_grouped_fp8_nt_contiguous((aq.to(torch.float8_e4m3fn).to(dev), sa.to(dev)),
+                                (bq.to(torch.float8_e4m3fn).to(dev), sb.to(dev)),
+                                torch.tensor(sizes, dtype=torch.int32, device=dev), out=out, grouped_layout=lay.to(dev))
+    out = out.cpu()
+    valid = lay >= 0
+    ad = (aq * sa.repeat_interleave(128, dim=1))[valid]
+    wd = bq * sb.repeat_interleave(128, dim=1).repeat_interleave(128, dim=2)
+    ref = torch.einsum("rk,rnk->rn", ad, wd[lay[valid].long()]).to(torch.bfloat16)
+    assert torch.equal(out[valid], ref)
+    assert bool((out[~valid] == 9.0).all()), "padding rows were written"
+
+
 def test_fp8_matrix_instruction_truncates_products_below_2_to_minus_13_of_the_largest(dev, variant):
     """Characterisation of gfx950's FP8 MFMA that the FP8 tolerances rest on: within one instruction the products
     are aligned to the largest one and bits below 2^-13 of it are dropped (truncated, not rounded), while the

@@ -92,13 +92,27 @@ def test_placement_from_per_row_layout_in_any_expert_order():
     # a per-row layout whose experts are not in ascending order: rows per expert and their first row, by hand
     from triton_grouped_gemm_amd.gemm.deep_gemm_ops import placement_from_layout
     lay = torch.tensor([2, 2, 2, -1, 0, 0, -1, -1, 3, -1, -1, -1], dtype=torch.int32)  # block_m = 4; expert 1 absent
-    rows, first = placement_from_layout(lay, 4)
-    assert rows.tolist() == [2, 0, 3, 1] and first.tolist() == [4, 0, 0, 8]
+    rows, first, expert = placement_from_layout(lay, 4)
+    assert rows.tolist() == [2, 0, 3, 1] and first.tolist() == [4, 0, 0, 8] and expert is None
     assert rows.dtype == torch.int32 and first.dtype == torch.int32
     # ascending layouts give the padded starts the builders use
     sizes = [128, 1, 127, 256, 0]
-    rows, first = placement_from_layout(L.make_deep_gemm_grouped_layout(sizes), len(sizes))
-    assert rows.tolist() == sizes and first.tolist() == [0, 128, 256, 384, 0]
+    rows, first, expert = placement_from_layout(L.make_deep_gemm_grouped_layout(sizes), len(sizes))
+    assert rows.tolist() == sizes and first.tolist() == [0, 128, 256, 384, 0] and expert is None
+
+
+def test_placement_from_per_row_layout_with_an_expert_in_several_regions():
+    # expert 2 owns rows 0..3 and 8..9, expert 0 rows 4..5 and row 11: one entry per region, in row order, by hand
+    from triton_grouped_gemm_amd.gemm.deep_gemm_ops import placement_from_layout
+    lay = torch.tensor([2, 2, 2, 2, 0, 0, -1, -1, 2, 2, -1, 0], dtype=torch.int64)
+    rows, first, expert = placement_from_layout(lay, 3)
+    assert rows.tolist() == [4, 2, 2, 1] and first.tolist() == [0, 4, 8, 11] and expert.tolist() == [2, 0, 2, 0]
+    assert rows.dtype == torch.int32 and first.dtype == torch.int32 and expert.dtype == torch.int64
+    # two regions of one expert that touch are one region; neighbours of different experts are two
+    rows, first, expert = placement_from_layout(torch.tensor([1, 1, 1, 1, 0, 0, 0, -1]), 2)
+    assert rows.tolist() == [3, 4] and first.tolist() == [4, 0] and expert is None
+    with pytest.raises(ValueError, match="beyond the 2"):
+        placement_from_layout(torch.tensor([0, 0, 2, -1]), 2)
 
 
 def test_reference_named_helpers():

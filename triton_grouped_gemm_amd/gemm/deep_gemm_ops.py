@@ -14,8 +14,11 @@ the psum form ``[G]`` (``use_psum_layout=True``: end offset of every expert's va
 ``block_m``) is differenced -- it places expert g after expert g-1 by construction; of the per-row form
 ``[M_padded]`` (expert id per row, -1 on padding rows) the rows of every expert are counted and their first row
 is located, so the experts' regions may follow one another in any order (``make_deep_gemm_grouped_layout``
-builds them ascending; a router that fills the buffer in arrival order does not).  One restriction remains: an
-expert's valid rows must be contiguous (one region per expert).
+builds them ascending; a router that fills the buffer in arrival order does not).  An expert whose rows lie in
+several separate regions is served as well, region by region: such a layout is recognised by one read-back of two
+counters (the wrappers already wait for the device once, for the reference's check of M) and the weights of the
+regions' experts are gathered into a temporary ``[regions, N, K]`` tensor for the call.  While a stream is being
+captured no read-back is possible and every expert is taken to have one region.
 """
 from __future__ import annotations
 
@@ -71,19 +74,44 @@ def sizes_from_layout(grouped_layout: torch.Tensor, num_groups: int, block_m: in
     return counts[1:].to(torch.int32)
 
 
-def placement_from_layout(grouped_layout: torch.Tensor, num_groups: int) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Per-row layout ``[M_padded]`` (expert id per row, -1 = padding) -> ``(rows, first_row)``, both int32 ``[G]``
-    on the layout's device, computed without a host round trip: how many rows carry expert id g and the smallest
-    such row index (0 for experts without rows).  Reference contract: gemm/layout.py:73-97 builds such layouts in
-    ascending expert order, gemm/deep_gemm_ops.py:24-100 forwards whatever the caller passes."""
+def placement_from_layout(grouped_layout: torch.Tensor, num_groups: int
+                          ) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """Per-row layout ``[M_padded]`` (expert id per row, -1 = padding) -> ``(rows, first_row, expert)``.
+
+    Every expert's rows in one region (the usual case): rows and first_row are int32 ``[G]`` on the layout's device
+    -- how many rows carry expert id g and the smallest such row index (0 for experts without rows) -- and expert
+    is None.  Some expert's rows in several regions: one entry per region (maximal run of rows with the same
+    non-negative id) in row order, and expert ``[regions]`` (int64) names the expert of each, for the caller to
+    gather the weights by.  Telling the two cases apart takes one read-back of two counters; while the current
+    stream is being captured it is left out and the first form is returned.  Reference contract:
+    gemm/layout.py:73-97 builds such layouts in ascending expert order, gemm/deep_gemm_ops.py:24-100 forwards
+    whatever the caller passes.
+    """
     lay = grouped_layout.to(torch.int64)
     m = lay.shape[0]
-    counts = torch.zeros(num_groups + 1, dtype=torch.int64, device=lay.device)
+    dev = lay.device
+    if m and not (lay.is_cuda and torch.cuda.is_current_stream_capturing()):
+        change = torch.ones(m, dtype=torch.bool, device=dev)
+        change[1:] = lay[1:] != lay[:-1]
+        seen = torch.zeros(num_groups + 1, dtype=torch.bool, device=dev)  # last slot: padding and ids out of range
+        seen[torch.where((lay >= 0) & (lay < num_groups), lay, num_groups)] = True
+        n_regions, n_experts, n_bad = torch.stack([(change & (lay >= 0)).sum(), seen[:num_groups].sum(),
+                                                   (lay >= num_groups).sum()]).tolist()
+        if n_bad:
+            raise ValueError(f"grouped_layout names experts beyond the {num_groups} that b holds")
+        if n_regions > n_experts:
+            if n_regions > _native.MAX_GROUPS:
+                raise ValueError(f"grouped_layout has {n_regions} separate regions, at most {_native.MAX_GROUPS} are supported")
+            starts = torch.nonzero(change).flatten()
+            lengths = torch.diff(starts, append=starts.new_tensor([m]))
+            keep = lay[starts] >= 0
+            return lengths[keep].to(torch.int32), starts[keep].to(torch.int32), lay[starts][keep]
+    counts = torch.zeros(num_groups + 1, dtype=torch.int64, device=dev)
     counts.scatter_add_(0, lay + 1, torch.ones_like(lay))
-    first = torch.full((num_groups + 1,), m, dtype=torch.int64, device=lay.device)
-    first.scatter_reduce_(0, lay + 1, torch.arange(m, dtype=torch.int64, device=lay.device), reduce="amin")
+    first = torch.full((num_groups + 1,), m, dtype=torch.int64, device=dev)
+    first.scatter_reduce_(0, lay + 1, torch.arange(m, dtype=torch.int64, device=dev), reduce="amin")
     first = torch.where(counts > 0, first, torch.zeros_like(first))
-    return counts[1:].to(torch.int32), first[1:].to(torch.int32)
+    return counts[1:].to(torch.int32), first[1:].to(torch.int32), None
 
 
 def m_grouped_bf16_nt_contiguous(a: torch.Tensor, b: torch.Tensor, size_per_group: torch.Tensor, *,
@@ -100,9 +128,11 @@ def m_grouped_bf16_nt_contiguous(a: torch.Tensor, b: torch.Tensor, size_per_grou
     if not (a.is_contiguous() and b.is_contiguous() and out.is_contiguous()):
         raise ValueError("a, b and out must be contiguous")
     if grouped_layout is not None and not use_psum_layout:  # per-row form: experts' regions in any order
-        rows, first = placement_from_layout(grouped_layout.to(a.device), g)
+        rows, first, expert = placement_from_layout(grouped_layout.to(a.device), g)
+        if expert is not None:  # an expert in several regions: one group per region, weights gathered to match
+            b = b.index_select(0, expert)
         _native.call("tgg_m_grouped_gemm_placed", a.data_ptr(), b.data_ptr(), out.data_ptr(), rows.data_ptr(), 0,
-                     first.data_ptr(), g, m, n, k, _native.BF16, -1, _native.stream_of(a))
+                     first.data_ptr(), rows.numel(), m, n, k, _native.BF16, -1, _native.stream_of(a))
         return out
     placed = size_per_group if grouped_layout is None else sizes_from_layout(grouped_layout, g, block_m, use_psum_layout)
     sizes, is64 = _sizes_on_device(placed, a.device)
@@ -152,9 +182,12 @@ def m_grouped_fp8_nt_contiguous(a: Tuple[torch.Tensor, torch.Tensor], b: Tuple[t
         sa = sa.t().contiguous().t()
     sb = b_scale.to(torch.float32).contiguous()
     if grouped_layout is not None and not use_psum_layout:  # per-row form: experts' regions in any order
-        rows, first = placement_from_layout(grouped_layout.to(a_codes.device), g)
+        rows, first, expert = placement_from_layout(grouped_layout.to(a_codes.device), g)
+        if expert is not None:  # an expert in several regions: one group per region, weights gathered to match
+            b_codes = b_codes.view(torch.uint8).index_select(0, expert)
+            sb = sb.index_select(0, expert)
         _native.call("tgg_m_grouped_gemm_fp8_block_placed", a_codes.data_ptr(), sa.data_ptr(), b_codes.data_ptr(),
-                     sb.data_ptr(), out.data_ptr(), rows.data_ptr(), 0, first.data_ptr(), g, m, n, k, 1, -1,
+                     sb.data_ptr(), out.data_ptr(), rows.data_ptr(), 0, first.data_ptr(), rows.numel(), m, n, k, 1, -1,
                      _native.stream_of(a_codes))
         return out
     placed = size_per_group if grouped_layout is None else sizes_from_layout(grouped_layout, g, block_m, use_psum_layout)
