@@ -1,14 +1,17 @@
 """Wait-state hazards around the inline-assembly memory instructions of the HIP kernels.
 
 The compiler inserts the wait states gfx9-family hardware needs between certain instruction pairs, but it does not
-look inside inline assembly.  Two of those pairs involve the hand-written vector-memory instructions of the tuned
+look inside inline assembly.  Three of those pairs involve the hand-written vector-memory instructions of the tuned
 kernels (direct-to-LDS copies, non-temporal stores):
   * a vector instruction writes a scalar register (v_readlane / v_readfirstlane, e.g. the reload of a spilled scalar)
     and a vector-memory instruction reads that register fewer than five wait states later: it sees the old value --
     for a buffer descriptor that means a wild address;
   * a 12- or 16-byte store is followed within two wait states by a vector instruction that overwrites its data
-    registers: the store writes the new value.
-Both were met while developing these kernels (a GPU memory fault, and wrong dwords in the output).  The build keeps
+    registers: the store writes the new value;
+  * a scalar instruction writes m0 and the very next instruction is a copy to LDS (a buffer load with the lds
+    modifier), which takes its LDS address from m0: one wait state must lie between them.
+The first two were met while developing these kernels (a GPU memory fault, and wrong dwords in the output); the
+third is the rule the compiler applies to its own copies of this kind.  The build keeps
 the device assembly (triton_grouped_gemm_amd/build/*.gfx950.s); this test scans it.  The scanner itself is checked
 on hand-written snippets, so the file tests something even where the library has not been built.
 """
@@ -46,6 +49,10 @@ def scan(text: str):
         toks = [t.strip(",") for t in line.split()[1:]]
         if not op.startswith(("buffer_", "global_", "flat_", "scratch_")):
             continue
+        if op.startswith("buffer_load") and toks[-1] == "lds" and i > 0:
+            prev = code[i - 1].split()
+            if prev[0].startswith("s_") and len(prev) > 1 and prev[1].strip(",") == "m0":
+                bad.append((code[i - 1], line, 0))
         need = set().union(*[_regs(t, "s") for t in toks]) if toks else set()
         ws = 0
         for d in range(1, 8):
@@ -89,6 +96,14 @@ def test_scanner_finds_overwritten_store_data():
     assert scan("global_store_dwordx4 v[8:9], v[0:3], off nt\ns_nop 1\nv_add_u32_e32 v0, 64, v8\n") == []
     assert scan("global_store_dwordx4 v[8:9], v[0:3], off nt\nv_add_u32_e32 v12, 64, v8\nv_mov_b32_e32 v13, v1\nv_mov_b32_e32 v0, v1\n") == []
     assert scan("global_store_dwordx2 v[8:9], v[0:1], off\nv_add_u32_e32 v0, 64, v8\n") == []  # 8-byte stores are not affected
+
+
+def test_scanner_finds_copy_to_lds_right_after_a_write_of_m0():
+    assert len(scan("s_mov_b32 m0, s2\nbuffer_load_dwordx4 v2, s[44:47], 0 offen lds\n")) == 1
+    assert len(scan("s_add_u32 m0, s2, 16\nbuffer_load_dword v2, s[44:47], 0 offen lds\n")) == 1
+    assert scan("s_mov_b32 m0, s2\ns_nop 0\nbuffer_load_dwordx4 v2, s[44:47], 0 offen lds\n") == []
+    assert scan("s_mov_b32 m0, s2\nv_add_u32_e32 v2, 64, v8\nbuffer_load_dwordx4 v2, s[44:47], 0 offen lds\n") == []
+    assert scan("s_mov_b32 m0, s2\nbuffer_load_dwordx4 v[2:5], v1, s[44:47], 0 offen\n") == []  # an ordinary load does not read m0
 
 
 def test_built_kernels_have_no_unspaced_hazard():

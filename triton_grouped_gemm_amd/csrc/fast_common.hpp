@@ -22,9 +22,11 @@ TGG_DEV void wait_vmcnt0_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(7 << 4); }
 // global source is the descriptor base + voff (bounds-checked: out-of-range lanes write zeros).
 // Written as inline assembly on purpose: the compiler does not model the copy, so it cannot
 // serialise the software pipeline with conservative waits; completion is tracked by hand with
-// wait_vmcnt<>() and the workgroup barrier.
+// wait_vmcnt<>() and the workgroup barrier.  s_nop 0: a copy to LDS that follows a scalar write of m0 needs one wait
+// state in between on this hardware generation (the compiler inserts it for its own such copies and does not look
+// inside this statement).
 TGG_DEV void copy_b128_to_lds(i32x4_t rsrc, uint32_t lds_addr, int voff) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" : : "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory", "m0");
 }
 
 // Output store of the tuned kernels; dst is global memory.  nt = non-temporal: the output is written once and

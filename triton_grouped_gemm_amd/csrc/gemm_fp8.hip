@@ -25,9 +25,9 @@ namespace {
 enum : int { EPI_CHANNEL = 1, EPI_BLOCK = 2 };
 constexpr int BKB = 128;  // K depth of a slab in fp8 values (= bytes)
 
-// One copy of 4 bytes per lane global -> LDS (destination m0 + lane * 4).
+// One copy of 4 bytes per lane global -> LDS (destination m0 + lane * 4; s_nop 0 as in copy_b128_to_lds).
 TGG_DEV void copy_b32_to_lds(i32x4_t rsrc, uint32_t lds_addr, int voff) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds" : : "s"(lds_addr), "v"(voff), "s"(rsrc) : "memory", "m0");
 }
 
 // BST: slab buffers of the B operand.  2: the A slab, the B slab and the activation scales of a stage sit together, two
