@@ -25,7 +25,9 @@ extern "C" {
 #define TGG_E4M3 2 /* OCP float8_e4m3fn */
 #define TGG_E5M2 3 /* OCP float8_e5m2 */
 
-#define TGG_MAX_GROUPS 1024
+#define TGG_MAX_GROUPS 1024      /* tgg_m_grouped_gemm, tgg_k_grouped_gemm(_queued); the quantizer's and the sort's tables */
+#define TGG_MAX_GROUPS_OTHER 512 /* every other GEMM entry point (padded, placed, masked, fused FP8 output, FP8): larger
+                                  * group counts are rejected with return code 1 */
 
 /* C[r,:] = A[r,:] . B[g(r)]^T (trans_b=1, B is [G,N,K]) or A[r,:] . B[g(r)] (trans_b=0, B is [G,K,N]);
  * rows of group g are the sizes[g] rows after those of groups < g; fp32 accumulate, output in `dtype`.

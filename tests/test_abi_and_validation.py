@@ -50,6 +50,33 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert lib.tgg_set_option(b"force_generic", 0) == 0
 
 
+def test_group_count_limits_per_entry_point():
+    """More than 512 groups are taken by the plain 16-bit M-grouped and K-grouped entry points only (up to 1024: the
+    shape-agnostic kernel serves them and is exercised there on the GPU); every other GEMM entry point rejects
+    them before anything is launched."""
+    lib = _native.load()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.addressof(buf)
+    p += (-p) % 16
+    calls = [
+        lambda g: lib.tgg_m_grouped_gemm_padded(p, p, p, p, 0, g, 1024, 128, 128, 128, 0, -1, None),
+        lambda g: lib.tgg_m_grouped_gemm_placed(p, p, p, p, 0, p, g, 1024, 128, 128, 0, -1, None),
+        lambda g: lib.tgg_m_grouped_gemm_masked(p, p, p, p, 0, g, 128, 1024, 128, 128, 1, 0, -1, None),
+        lambda g: lib.tgg_m_grouped_gemm_fp8_out(p, p, p, p, p, 0, g, 1024, 128, 128, 1, 0, 2, 0, -1, None),
+        lambda g: lib.tgg_m_grouped_gemm_fp8_channel(p, p, p, p, p, p, 0, g, 1024, 128, 128, 2, 2, 0, -1, None),
+        lambda g: lib.tgg_k_grouped_gemm_fp8_channel(p, p, p, p, p, p, g, 128, 128, 1024, 2, 2, -1, None),
+        lambda g: lib.tgg_m_grouped_gemm_fp8_block(p, p, p, p, p, p, 0, g, 1024, 128, 128, 128, 1, -1, None),
+        lambda g: lib.tgg_m_grouped_gemm_fp8_block_placed(p, p, p, p, p, p, 0, p, g, 1024, 128, 128, 1, -1, None),
+    ]
+    for call in calls:
+        assert call(_native.MAX_GROUPS_OTHER + 1) == 1
+        assert f"G=513 outside [1, {_native.MAX_GROUPS_OTHER}]" in _native.last_error()
+    assert lib.tgg_m_grouped_gemm(p, p, p, p, 0, _native.MAX_GROUPS + 1, 128, 128, 128, 1, 0, -1, None) == 1
+    assert "G=1025 outside [1, 1024]" in _native.last_error()
+    assert lib.tgg_k_grouped_gemm(p, p, p, p, p, _native.MAX_GROUPS + 1, 128, 128, 1024, 0, -1, None) == 1
+    assert "G=1025 outside [1, 1024]" in _native.last_error()
+
+
 def test_reference_import_paths_resolve():
     tgg.install_aliases()
     from gemm.BF16.m_grouped_gemm_TMA import m_grouped_gemm, _build_m_grouped_metadata, _m_grouped_gemm_launch  # noqa

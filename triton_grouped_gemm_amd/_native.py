@@ -14,7 +14,8 @@ import torch
 LIB_PATH = Path(__file__).resolve().parent / "libtgg_amd.so"
 
 BF16, F16, E4M3, E5M2 = 0, 1, 2, 3
-MAX_GROUPS = 1024
+MAX_GROUPS = 1024  # TGG_MAX_GROUPS: plain 16-bit M-grouped and K-grouped GEMM
+MAX_GROUPS_OTHER = 512  # TGG_MAX_GROUPS_OTHER: every other GEMM entry point
 QUEUE_WORDS = 8  # TGG_QUEUE_WORDS: int32 counters of the K-grouped kernels' work queue
 
 _P, _I, _L = c_void_p, c_int, c_int64

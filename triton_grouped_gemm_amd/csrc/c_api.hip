@@ -60,10 +60,13 @@ void set_fp8_variant(int v);
 
 static bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
 
-static int check_common(const void* A, const void* B, const void* C, const void* sizes, int G, int N) {
+// max_groups: TGG_MAX_GROUPS for the two plain 16-bit entry points (M-grouped, K-grouped), whose shape-agnostic
+// kernel is exercised on the GPU above 512 groups; TGG_MAX_GROUPS_OTHER for every other GEMM entry point.
+static int check_common(const void* A, const void* B, const void* C, const void* sizes, int G, int N,
+                        int max_groups = TGG_MAX_GROUPS_OTHER) {
   if (!A || !B || !C) return set_error("null operand pointer");
   if (!sizes) return set_error("null group-size pointer");
-  if (G < 1 || G > TGG_MAX_GROUPS) return set_error("G=%d outside [1, %d]", G, TGG_MAX_GROUPS);
+  if (G < 1 || G > max_groups) return set_error("G=%d outside [1, %d]", G, max_groups);
   if (N < 1) return set_error("N=%d must be positive", N);
   if (!aligned16(A) || !aligned16(B) || !aligned16(C)) return set_error("operand pointers must be 16-byte aligned");
   return 0;
@@ -125,7 +128,7 @@ extern "C" {
 
 int tgg_m_grouped_gemm(const void* A, const void* B, void* C, const void* sizes, int sizes_i64, int G, int64_t M,
                        int N, int K, int trans_b, int dtype, int num_cu, void* stream) {
-  if (int e = check_common(A, B, C, sizes, G, N)) return e;
+  if (int e = check_common(A, B, C, sizes, G, N, TGG_MAX_GROUPS)) return e;
   if (M < 0 || K < 0) return set_error("negative M or K");
   if (dtype != TGG_BF16 && dtype != TGG_F16) return set_error("data type code %d not supported", dtype);
   if ((K & 7) || (N & 7)) return set_error("N and K must be multiples of 8 (16-byte rows), got N=%d K=%d", N, K);
@@ -225,7 +228,7 @@ int tgg_k_grouped_gemm(const void* A, const void* B, void* C, const int32_t* sta
 
 int tgg_k_grouped_gemm_queued(const void* A, const void* B, void* C, const int32_t* start, const int32_t* end, int G,
                               int Mdim, int N, int64_t Ktot, int dtype, int num_cu, int32_t* queue, void* stream) {
-  if (int e = check_common(A, B, C, start, G, N)) return e;
+  if (int e = check_common(A, B, C, start, G, N, TGG_MAX_GROUPS)) return e;
   if (!end) return set_error("null group_end pointer");
   if (Mdim < 1 || Ktot < 0) return set_error("bad Mdim=%d or Ktot=%lld", Mdim, (long long)Ktot);
   if (dtype != TGG_BF16 && dtype != TGG_F16) return set_error("data type code %d not supported", dtype);

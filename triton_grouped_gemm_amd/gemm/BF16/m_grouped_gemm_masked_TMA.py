@@ -35,7 +35,7 @@ def m_grouped_gemm_masked(lhs: Tensor, rhs: Tensor, out: Tensor, masked_m: Tenso
     assert out.dim() == 2 and tuple(out.shape) == (M, N), "out should have shape [M, N]"
     assert masked_m.dim() == 1 and masked_m.shape[0] == num_groups, "masked_m must hold one entry per group"
     assert num_groups * int(expected_m) <= M, "expected_m * num_groups must not exceed the rows of lhs"
-    assert num_groups <= _native.MAX_GROUPS, f"at most {_native.MAX_GROUPS} groups are supported"
+    assert num_groups <= _native.MAX_GROUPS_OTHER, f"at most {_native.MAX_GROUPS_OTHER} groups are supported"
     _native.require_gpu(lhs, rhs, out)
     assert lhs.is_contiguous() and rhs.is_contiguous() and out.is_contiguous(), "lhs, rhs and out must be contiguous"
     mm, is64 = _sizes_on_device(masked_m, lhs.device)

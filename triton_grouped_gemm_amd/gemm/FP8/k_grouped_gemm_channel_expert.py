@@ -34,7 +34,7 @@ def matmul(x_fp8: Tensor, x_scale: Tensor, y_fp8: Tensor, y_scale: Tensor, token
     assert y_fp8.dim() == 2 and tuple(y_fp8.shape) == (N, K), "y_fp8 must be [N, K]"
     assert x_fp8.element_size() == 1 and y_fp8.element_size() == 1, "x_fp8 and y_fp8 must hold 8-bit codes"
     assert tokens_per_expert.dim() == 1 and tokens_per_expert.shape[0] == num_groups
-    assert 1 <= num_groups <= _native.MAX_GROUPS, f"between 1 and {_native.MAX_GROUPS} groups are supported"
+    assert 1 <= num_groups <= _native.MAX_GROUPS_OTHER, f"between 1 and {_native.MAX_GROUPS_OTHER} groups are supported"
     _native.require_gpu(x_fp8, x_scale, y_fp8, y_scale)
     assert x_fp8.is_contiguous() and y_fp8.is_contiguous(), "x_fp8 and y_fp8 must be contiguous"
     xs = _expert_major(x_scale, M, num_groups)

@@ -31,7 +31,7 @@ def gmm_fp8_act_per_channel_w_per_expert(A: Tensor, A_scale: Tensor, B: Tensor, 
     assert dtype_out in _native.DTYPE_CODE, f"data type {dtype_out} not supported"
     assert A_scale.numel() == M and B_scale.numel() == num_groups * N, "scale tensors have the wrong number of entries"
     assert size_per_group.dim() == 1 and size_per_group.shape[0] == num_groups
-    assert num_groups <= _native.MAX_GROUPS, f"at most {_native.MAX_GROUPS} groups are supported"
+    assert num_groups <= _native.MAX_GROUPS_OTHER, f"at most {_native.MAX_GROUPS_OTHER} groups are supported"
     _native.require_gpu(A, A_scale, B, B_scale)
     assert A.is_contiguous() and B.is_contiguous(), "A and B must be contiguous"
     a_s = A_scale.to(torch.float32).contiguous()

@@ -100,8 +100,8 @@ def placement_from_layout(grouped_layout: torch.Tensor, num_groups: int
         if n_bad:
             raise ValueError(f"grouped_layout names experts beyond the {num_groups} that b holds")
         if n_regions > n_experts:
-            if n_regions > _native.MAX_GROUPS:
-                raise ValueError(f"grouped_layout has {n_regions} separate regions, at most {_native.MAX_GROUPS} are supported")
+            if n_regions > _native.MAX_GROUPS_OTHER:
+                raise ValueError(f"grouped_layout has {n_regions} separate regions, at most {_native.MAX_GROUPS_OTHER} are supported")
             starts = torch.nonzero(change).flatten()
             lengths = torch.diff(starts, append=starts.new_tensor([m]))
             keep = lay[starts] >= 0
