@@ -67,12 +67,13 @@ int tgg_k_grouped_gemm(const void* A, const void* B, void* C, const int32_t* sta
 /* tgg_k_grouped_gemm with a work queue (same reference function, gemm/BF16/k_grouped_gemm_TMA.py:217-294).  A
  * K-grouped tile costs what its group has tokens, so with ragged groups no fixed assignment of tiles to the
  * persistent workgroups is even.  `queue` points to TGG_QUEUE_WORDS int32 in device memory that are ZERO when the
- * kernel starts (clear them on the same stream, with a fill kernel if the call may be captured into a graph); the
- * workgroups draw their tile ids from them (one counter per XCD), largest groups first, and a workgroup that drew
- * expensive tiles draws fewer.  Results are bit-identical to tgg_k_grouped_gemm; the kernel leaves the counters at
- * the numbers of ids drawn.  A launch must have the words to itself until it has finished.  queue = NULL: the
- * fixed assignment. */
-#define TGG_QUEUE_WORDS 8
+ * kernel starts; the workgroups draw their tile ids from them (one counter per XCD), largest groups first, and a
+ * workgroup that drew expensive tiles draws fewer.  Results are bit-identical to tgg_k_grouped_gemm.  The kernel
+ * leaves the words ZERO again (the workgroup that finishes last clears them), so a caller clears them once, when it
+ * allocates them, and may pass the same words to launch after launch on one stream -- also inside a captured graph,
+ * with no fill node.  A launch must have the words to itself until it has finished (one queue per stream).
+ * queue = NULL: the fixed assignment. */
+#define TGG_QUEUE_WORDS 16 /* eight counters, the count of finished workgroups, seven spare */
 int tgg_k_grouped_gemm_queued(const void* A, const void* B, void* C, const int32_t* start, const int32_t* end, int G,
                               int Mdim, int N, int64_t Ktot, int dtype, int num_cu, int32_t* queue, void* stream);
 
@@ -91,8 +92,9 @@ int tgg_k_grouped_gemm_fp8_channel(const void* x, const float* xs, const void* y
                                    int num_cu, void* stream);
 
 /* tgg_k_grouped_gemm_fp8_channel with a work queue (same reference function,
- * gemm/FP8/k_grouped_gemm_channel_expert.py:143-181); `queue` as in tgg_k_grouped_gemm_queued.  Only the tuned
- * kernel (token counts that are all multiples of 16) draws from it; the shape-agnostic kernel leaves it untouched. */
+ * gemm/FP8/k_grouped_gemm_channel_expert.py:143-181); `queue` as in tgg_k_grouped_gemm_queued (zero before, zero
+ * after).  Only the tuned kernel (token counts that are all multiples of 16) draws from it; the shape-agnostic
+ * kernel leaves it untouched. */
 int tgg_k_grouped_gemm_fp8_channel_queued(const void* x, const float* xs, const void* y, const float* ys, void* out,
                                           const int32_t* tokens, int G, int M, int N, int64_t Ktot, int fmt_a,
                                           int fmt_b, int num_cu, int32_t* queue, void* stream);
@@ -205,6 +207,19 @@ int tgg_debug_tile_order(const int64_t* sizes, int G, int mode, int64_t m_total,
 int tgg_debug_row_tiles(const int64_t* sizes, int G, int mode, int64_t m_total, int64_t aux, int tile, int n_chunk,
                         int64_t* out, int64_t capacity, int64_t* num_row_tiles);
 
+/* Test hook, host only: which elements of each operand the shape-agnostic kernel would touch for a launch of the
+ * given entry point, found by walking every tile with the kernel's own scheduler and address arithmetic.  It guards
+ * what the reference gets from Triton's masked loads and TMA bounds (e.g. gemm/BF16/m_grouped_gemm.py:83-116,
+ * gemm/FP8/m_grouped_gemm_channel_expert.py:119-136): no access outside the tensors, whatever the group count.
+ *   kind  0 / 1 tgg_m_grouped_gemm with trans_b = 1 / 0; 2 masked (aux = m_stride); 3 padded (aux = align);
+ *         4 placed (row_start); 5 tgg_k_grouped_gemm (sizes = token counts, M = Mdim, aux = Ktot);
+ *         6 FP8 per-channel M-grouped; 7 FP8 per-channel K-grouped (M = rows of x, aux = Ktot);
+ *         8 / 9 FP8 block-scaled with sa stored [M, KB] / [KB, M] (aux = align); 10 the same, placed (row_start)
+ *   out   [7][2] = lowest and highest element index touched in A, B, C, scale_m, scale_n, sa, sb
+ *         ({INT64_MAX, -1} for an operand that is never touched) */
+int tgg_debug_generic_extents(int kind, const int64_t* sizes, const int32_t* row_start, int G, int64_t M, int64_t aux,
+                              int N, int K, int64_t* out);
+
 /* Test hook, host only: the deal of the K-grouped kernels' work queue.  out[xq][n] (row-major, [8][draws]) = the tile
  * id behind the n-th draw from XCD xq's counter on a grid of `grid` workgroups (a multiple of 8; other grids use
  * one counter whose draws are the ids themselves).  The reference has no counterpart (its K-grouped kernels walk
@@ -212,7 +227,9 @@ int tgg_debug_row_tiles(const int64_t* sizes, int G, int mode, int64_t m_total, 
  * together list every id once and each of them in growing order. */
 int tgg_debug_queue_order(int grid, int draws, int32_t* out);
 
-/* Library controls (process-wide, meant for tests and tuning; returns 1 for an unknown key):
+/* Library controls (process-wide test and tuning hooks, not a per-call interface: every launch reads each option
+ * once, atomically, so a thread that changes one while another thread launches decides only which value that launch
+ * sees; returns 1 for an unknown key):
  *   "force_generic" 0/1  route every GEMM through the shape-agnostic kernel
  *   "variant"       int  tile configuration of the tuned kernels (16-bit, and FP8 M-grouped): 0 (default) = chosen per launch on the
  *                        device from the group sizes -- 256x128 when all such tiles fit one round of the persistent

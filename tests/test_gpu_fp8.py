@@ -207,7 +207,11 @@ def test_fp8_k_grouped_work_queue_equals_fixed_assignment(dev, tokens):
                  drawn.data_ptr(), tok.data_ptr(), G, M, N, Kt, _native.E4M3, _native.E4M3, -1, queue.data_ptr(), st)
     assert not bool(torch.isnan(fixed.float()).any())
     assert torch.equal(fixed, drawn)
-    assert int(queue.sum()) >= G * ((M + 255) // 256) * ((N + 255) // 256)
+    assert int(queue.abs().sum()) == 0, "the last workgroup clears the queue"
+    drawn.fill_(float("nan"))
+    _native.call("tgg_k_grouped_gemm_fp8_channel_queued", x.data_ptr(), xs_t.data_ptr(), y.data_ptr(), ys_t.data_ptr(),
+                 drawn.data_ptr(), tok.data_ptr(), G, M, N, Kt, _native.E4M3, _native.E4M3, -1, queue.data_ptr(), st)
+    assert torch.equal(fixed, drawn), "second launch on the same, uncleared words"
 
 
 def _block_scaled_case(sizes, N, K, seed):

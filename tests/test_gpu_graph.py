@@ -147,9 +147,10 @@ def test_deep_gemm_shaped_wrappers_can_be_captured(dev):
 
 
 def test_k_grouped_wrapper_with_its_work_queue_can_be_captured(dev):
-    """k_grouped_gemm clears the kernel's tile counters with a small fill kernel on every call; captured, that fill is
-    part of the graph, so every replay starts from zero counters.  Replays with other token counts (read on the
-    device) must equal the eager call."""
+    """The K-grouped kernel finds its tile counters zero and leaves them zero.  A capture without a caller-owned queue
+    gets a fresh zeroed tensor whose fill is part of the graph; with ``queue=`` the graph holds the GEMM kernel alone
+    and nothing is allocated inside the call.  Replays with other token counts (read on the device) must equal the
+    eager call."""
     G, Kt, Mdim, N = 6, 3072, 264, 520
     a, b = _randn((Kt, Mdim), 41, dev), _randn((Kt, N), 42, dev)
     sizes = torch.tensor([512] * G, dtype=torch.int32, device=dev)
@@ -164,3 +165,16 @@ def test_k_grouped_wrapper_with_its_work_queue_can_be_captured(dev):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, k_grouped_gemm(a, b, sizes)), f"replay {it}"
+    from triton_grouped_gemm_amd import _native
+    queue = torch.zeros(_native.QUEUE_WORDS, dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()
+    graph2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph2):
+        out2 = k_grouped_gemm(a, b, sizes, queue=queue)
+    for it, routing in enumerate([[3000, 0, 0, 8, 0, 64], [512] * G, [0, 1024, 1024, 0, 1000, 24]]):
+        sizes.copy_(torch.tensor(routing, dtype=torch.int32))
+        torch.cuda.synchronize()
+        graph2.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out2, k_grouped_gemm(a, b, sizes)), f"caller-owned queue, replay {it}"
+        assert int(queue.abs().sum()) == 0

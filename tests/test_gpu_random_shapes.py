@@ -272,3 +272,41 @@ def test_non_finite_inputs_stay_in_their_row_and_column(dev):
     expect_bad[429:, 77] = True       # group 3 holds rows 429..1128
     assert bool((~torch.isfinite(out.float()) == expect_bad).all())
     assert torch.equal(out[~expect_bad], clean[~expect_bad])
+
+
+@pytest.mark.skip(reason="masked / padded / FP8 entry points reject more than 512 groups (TGG_MAX_GROUPS_OTHER): the one GPU run "
+                         "that held these cases ended in a GPU fault whose cause has not been shown, so they stay off the GPU. "
+                         "The host-side walks in tests/test_generic_bounds.py and tests/test_tile_order.py cover the "
+                         "shape-agnostic kernel's scheduler and addressing up to 1024 groups.")
+@pytest.mark.parametrize("G", [513, 700, 1024])
+def test_more_than_512_groups_on_the_other_entry_points(dev, G):
+    """What would be checked once the limit is lifted: masked, FP8 per-channel, FP8 block-scaled and FP8 K-grouped
+    problems with more than 512 groups against torch's fp32 product, group by group."""
+    from oracle import gemm_ref
+    from triton_grouped_gemm_amd.gemm.deep_gemm_ops import m_grouped_fp8_nt_contiguous
+    from triton_grouped_gemm_amd.quant.fp8_cast import per_block_cast_to_fp8, per_token_cast_to_fp8
+    rng = random.Random(G)
+    sizes = [rng.choice([0, 0, 3, 16, 40, 128, 129, 300]) for _ in range(G)]
+    sizes[511], sizes[512] = 77, 130
+    N, K = 264, 136
+    torch.manual_seed(G)
+    b = torch.randn(G, N, K, device=dev).to(torch.bfloat16)
+    m_max = 256
+    mm = torch.tensor([rng.randint(0, m_max) for _ in range(G)], dtype=torch.int32, device=dev)
+    am = (torch.randn(G * m_max, K, device=dev) * K ** -0.5).to(torch.bfloat16)
+    out = torch.full((G * m_max, N), 7.0, dtype=torch.bfloat16, device=dev)
+    m_grouped_gemm_masked(am, b, out, mm, m_max)
+    for g in range(G):
+        cnt = int(mm[g])
+        rows = out[g * m_max:g * m_max + cnt]
+        assert _half_ulp_of_fp32(rows, am[g * m_max:g * m_max + cnt].float() @ b[g].float().t()), f"masked group {g}"
+        assert bool((out[g * m_max + cnt:(g + 1) * m_max] == 7.0).all())
+    padded = [(s + 127) // 128 * 128 for s in sizes]
+    ap = torch.randn(sum(padded), 256, device=dev).to(torch.bfloat16)
+    w = torch.randn(G, N, 256, device=dev).to(torch.bfloat16)
+    aq, sa = per_token_cast_to_fp8(ap, scales_mn_major=True)
+    wq, sb = per_block_cast_to_fp8(w)
+    st = torch.tensor(sizes, dtype=torch.int32, device=dev)
+    got = m_grouped_fp8_nt_contiguous((aq, sa), (wq, sb), st)
+    ref = gemm_ref.fp8_block_scaled_reference(aq.cpu().float(), sa.cpu(), wq.cpu().float(), sb.cpu(), sizes, 128)
+    assert gemm_ref.rdiff(got.cpu(), ref) <= 2e-2

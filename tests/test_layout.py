@@ -111,8 +111,18 @@ def test_placement_from_per_row_layout_with_an_expert_in_several_regions():
     # two regions of one expert that touch are one region; neighbours of different experts are two
     rows, first, expert = placement_from_layout(torch.tensor([1, 1, 1, 1, 0, 0, 0, -1]), 2)
     assert rows.tolist() == [3, 4] and first.tolist() == [4, 0] and expert is None
-    with pytest.raises(ValueError, match="beyond the 2"):
+    with pytest.raises(ValueError, match=r"outside \[-1, 2\)"):
         placement_from_layout(torch.tensor([0, 0, 2, -1]), 2)
+    with pytest.raises(ValueError, match=r"outside \[-1, 2\)"):
+        placement_from_layout(torch.tensor([0, 0, -3, -1]), 2)
+
+
+def test_layout_ids_that_name_no_expert_count_as_padding_where_nothing_can_be_checked():
+    """sizes_from_layout never reads back (it is what a captured call uses): ids below -1 or beyond the experts must
+    not index outside its table; their rows belong to no group."""
+    from triton_grouped_gemm_amd.gemm.deep_gemm_ops import sizes_from_layout
+    lay = torch.tensor([0, 0, 7, -1, 1, -5, 1, 1], dtype=torch.int32)
+    assert sizes_from_layout(lay, 2, 4, False).tolist() == [2, 3]
 
 
 def test_reference_named_helpers():

@@ -190,3 +190,59 @@ def test_work_queue_deals_every_tile_once_and_each_counter_in_growing_order(grid
         assert np.array_equal(order, np.arange(8) if k % 2 == 0 else np.arange(8)[::-1]), "back and forth"
     bad = np.zeros((8, 4), dtype=np.int32)
     assert lib.tgg_debug_queue_order(100, 4, bad.ctypes.data) == 1  # not a multiple of 8: one counter, ids in order
+
+
+def _many_group_sizes(G, seed, top):
+    rng = np.random.default_rng(seed)
+    sizes = rng.choice([0, 0, 3, 16, 40, 128, 129, 300, top], size=G)
+    sizes[G // 2 - 1], sizes[G // 2] = 77, 130  # rows on both sides of the middle of the table
+    sizes[511], sizes[512] = 77, 130             # ... and of entry 512
+    return [int(x) for x in sizes]
+
+
+@pytest.mark.parametrize("tile", [128, 256])
+@pytest.mark.parametrize("G", [513, 600, 1024])
+@pytest.mark.parametrize("mode", [MG, MG_PAD, MASKED, KG_COUNT])
+def test_cover_with_more_than_512_groups(tile, G, mode):
+    """Group counts beyond the tuned kernels' 512-entry table, which the shape-agnostic kernel's 1024-entry table
+    takes: every tile exactly once, rows inside each group's range and inside the operand, for every way the groups
+    can be laid out (contiguous, padded, masked, K-grouped by counts)."""
+    N, grid = 264, 256
+    if mode == MASKED:
+        m_stride = 256
+        sizes = _many_group_sizes(G, G + tile, m_stride)  # holds counts above m_stride: the kernel clips them
+        rows, n = tile_order(sizes, MASKED, G * m_stride, m_stride, N, tile, grid, 1)
+        starts = [g * m_stride for g in range(G)]
+        exp = expected_m_grouped_tiles([min(s, m_stride) for s in sizes], starts, tile, N, G * m_stride)
+    elif mode == KG_COUNT:
+        sizes = [16 * (s % 13) for s in _many_group_sizes(G, G + tile, 192)]
+        mdim = 136
+        rows, n = tile_order(sizes, KG_COUNT, mdim, sum(sizes), N, tile, grid, 0)
+        exp = {(g, mt * tile, min(tile, mdim - mt * tile), nt * tile)
+               for g in range(G) for mt in range(-(-mdim // tile)) for nt in range(-(-N // tile))}
+    else:
+        sizes = _many_group_sizes(G, G + tile, 517)
+        align = 128 if mode == MG_PAD else 1
+        padded = [-(-s // align) * align for s in sizes]
+        starts = np.concatenate([[0], np.cumsum(padded)[:-1]]).tolist()
+        m_total = sum(padded)
+        rows, n = tile_order(sizes, mode, m_total, align if mode == MG_PAD else 0, N, tile, grid, 1)
+        exp = expected_m_grouped_tiles(sizes, starts, tile, N, m_total)
+    got = [tuple(r[2:6]) for r in rows.tolist()]
+    assert n == len(exp) == len(got)
+    assert set(got) == exp and len(set(got)) == len(got)
+    assert 0 <= rows[:, 2].min() and rows[:, 2].max() < G
+
+
+def test_a_negative_row_start_gives_the_group_no_rows():
+    """Placed groups take their first row from device memory: a start in front of the operand must not be computed on
+    (the upper end was always clipped)."""
+    lib = _native.load()
+    sizes = np.asarray([100, 50, 30], dtype=np.int64)
+    starts = np.asarray([200, -64, 0], dtype=np.int32)
+    out = np.zeros((7, 2), dtype=np.int64)
+    assert lib.tgg_debug_generic_extents(4, sizes.ctypes.data, starts.ctypes.data, 3, 300, 0, 128, 64, out.ctypes.data) == 0
+    assert out[0, 0] == 0 and out[0, 1] == 299 * 64 + 63         # A: rows 0..29 and 200..299 only
+    assert out[2, 0] == 0 and out[2, 1] == 299 * 128 + 127       # C likewise
+    assert out[1, 0] == 0 and out[1, 1] == 3 * 128 * 64 - 1      # weights of groups 0 and 2 (group 1 is never touched,
+    #                                                              but it lies between them)

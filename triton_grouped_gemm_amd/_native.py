@@ -8,6 +8,7 @@ from __future__ import annotations
 import ctypes
 from ctypes import c_char_p, c_int, c_int64, c_void_p
 from pathlib import Path
+from typing import Optional
 
 import torch
 
@@ -16,7 +17,7 @@ LIB_PATH = Path(__file__).resolve().parent / "libtgg_amd.so"
 BF16, F16, E4M3, E5M2 = 0, 1, 2, 3
 MAX_GROUPS = 1024  # TGG_MAX_GROUPS: plain 16-bit M-grouped and K-grouped GEMM
 MAX_GROUPS_OTHER = 512  # TGG_MAX_GROUPS_OTHER: every other GEMM entry point
-QUEUE_WORDS = 8  # TGG_QUEUE_WORDS: int32 counters of the K-grouped kernels' work queue
+QUEUE_WORDS = 16  # TGG_QUEUE_WORDS: int32 words of the K-grouped kernels' work queue (zero before a launch, zero after)
 
 _P, _I, _L = c_void_p, c_int, c_int64
 
@@ -47,6 +48,7 @@ SIGNATURES = {
     "tgg_debug_tile_order": [_P, _I, _I, _L, _L, _I, _I, _I, _I, _P, _L, _P],
     "tgg_debug_row_tiles": [_P, _I, _I, _L, _L, _I, _I, _P, _L, _P],
     "tgg_debug_queue_order": [_I, _I, _P],
+    "tgg_debug_generic_extents": [_I, _P, _P, _I, _L, _L, _I, _I, _P],
     "tgg_set_option": [c_char_p, _I],
     "tgg_version": [],
 }
@@ -88,6 +90,29 @@ def set_option(key: str, value: int) -> None:
 
 def stream_of(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+_work_queues = {}
+
+
+def work_queue(device: torch.device, queue: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The K-grouped kernels' tile counters for a launch on ``device``'s current stream: the caller's ``queue``
+    (QUEUE_WORDS int32 on that device, zero, and not in use by a launch on another stream) or one the library keeps
+    per (device, stream).  The kernels leave the words zero again, so the kept tensor is cleared once, when it is
+    made, and a call costs no fill kernel and no allocation.  While the stream is being captured a tensor made here
+    would belong to the graph's memory pool: the capture gets a fresh one (its fill is part of the graph) unless
+    the caller brings its own."""
+    if queue is not None:
+        assert queue.is_cuda and queue.device == device and queue.dtype == torch.int32 and queue.is_contiguous() \
+            and queue.numel() >= QUEUE_WORDS, f"queue must be {QUEUE_WORDS} contiguous int32 on {device}"
+        return queue
+    if torch.cuda.is_current_stream_capturing():
+        return torch.zeros(QUEUE_WORDS, dtype=torch.int32, device=device)
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    q = _work_queues.get(key)
+    if q is None:
+        q = _work_queues[key] = torch.zeros(QUEUE_WORDS, dtype=torch.int32, device=device)
+    return q
 
 
 def ptr(t) -> int:

@@ -3,20 +3,26 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <atomic>
+#include <vector>
+
 #include "../../include/tgg_amd.h"
 #include "common.hpp"
+#include "generic_addr.hpp"
 #include "launch.hpp"
 #include "sched.hpp"
 
 namespace tgg {
 
 static thread_local char g_err[512] = "";
-static int g_force_generic = 0;
-static int g_tile_split = 1;
-static int g_store_nt = 1;
-static int g_n_chunk = 0;
-static int g_kg_second_launch = 1;
-static int g_four_wave = 0;  // 0 = eight-wave kernels only, 1 = four-wave kernel on large M-grouped NT launches, 2 = on every launch it can take
+// Process-wide options (tgg_set_option): test and tuning hooks.  Atomic so that a thread that flips one while another
+// thread launches is a race on which value that launch sees, not undefined behaviour; a launch reads each option once.
+static std::atomic<int> g_force_generic{0};
+static std::atomic<int> g_tile_split{1};
+static std::atomic<int> g_store_nt{1};
+static std::atomic<int> g_n_chunk{0};
+static std::atomic<int> g_kg_second_launch{1};
+static std::atomic<int> g_four_wave{0};  // 0 = eight-wave kernels only, 1 = four-wave kernel on large M-grouped NT launches, 2 = on every launch it can take
 
 int set_error(const char* fmt, ...) {
   va_list ap;
@@ -81,9 +87,97 @@ static GemmParams zero_params() {
   return p;
 }
 
+
+// GemmParams of each GEMM entry point, assembled in one place: the entry points launch with them and
+// tgg_debug_generic_extents walks the same parameter blocks on the host.
+static GemmParams params_m_grouped(const void* A, const void* B, void* C, const void* sizes, int sizes_i64, int G,
+                                   int64_t M, int N, int K, int trans_b, int num_cu) {
+  GemmParams p = zero_params();
+  p.A = A; p.B = B; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
+  p.mode = MODE_MG; p.m_total = M; p.N = N; p.K = K;
+  p.a_sm = K; p.a_sk = 1;
+  p.b_sg = (int64_t)N * K;
+  if (trans_b) { p.b_sn = K; p.b_sk = 1; } else { p.b_sn = 1; p.b_sk = N; }
+  p.grid_limit = num_cu;
+  return p;
+}
+
+// rows physically padded to `align` per group, or (row_start given) every group's rows at its own start
+static GemmParams params_padded(const void* A, const void* B, void* C, const void* sizes, int sizes_i64,
+                                const int32_t* row_start, int G, int64_t M, int N, int K, int align, int num_cu) {
+  GemmParams p = zero_params();
+  p.A = A; p.B = B; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
+  p.mode = MODE_MG_PAD; p.align = row_start ? 1 : align; p.row_start = row_start; p.m_total = M; p.N = N; p.K = K;
+  p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K; p.b_sn = K; p.b_sk = 1;
+  p.grid_limit = num_cu;
+  return p;
+}
+
+static GemmParams params_masked(const void* A, const void* B, void* C, const void* masked_m, int masked_i64, int G,
+                                int64_t m_stride, int64_t M, int N, int K, int trans_b, int num_cu) {
+  GemmParams p = zero_params();
+  p.A = A; p.B = B; p.C = C; p.sizes = masked_m; p.sizes_i64 = masked_i64; p.G = G;
+  p.mode = MODE_MASKED; p.m_stride = m_stride; p.m_total = M; p.N = N; p.K = K;
+  p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K;
+  if (trans_b) { p.b_sn = K; p.b_sk = 1; } else { p.b_sn = 1; p.b_sk = N; }
+  p.grid_limit = num_cu;
+  return p;
+}
+
+static GemmParams params_k_grouped(const void* A, const void* B, void* C, const int32_t* start, const int32_t* end,
+                                   int G, int Mdim, int N, int64_t Ktot, int num_cu, int32_t* queue) {
+  GemmParams p = zero_params();
+  p.A = A; p.B = B; p.C = C; p.k_start = start; p.k_end = end; p.G = G;
+  p.mode = MODE_KG; p.m_total = Mdim; p.k_total = Ktot; p.N = N; p.K = 0;
+  p.a_sm = 1; p.a_sk = Mdim; p.b_sg = 0; p.b_sn = 1; p.b_sk = N; p.c_sg = (int64_t)Mdim * N;
+  p.grid_limit = num_cu;
+  p.queue = queue;
+  return p;
+}
+
+static GemmParams params_fp8_channel(const void* Aq, const float* a_scale, const void* Bq, const float* b_scale,
+                                     void* C, const void* sizes, int sizes_i64, int G, int64_t M, int N, int K,
+                                     int num_cu) {
+  GemmParams p = zero_params();
+  p.A = Aq; p.B = Bq; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
+  p.scale_m = a_scale; p.scale_n = b_scale;
+  p.mode = MODE_MG; p.m_total = M; p.N = N; p.K = K;
+  p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K; p.b_sn = K; p.b_sk = 1;
+  p.grid_limit = num_cu;
+  return p;
+}
+
+static GemmParams params_fp8_k_channel(const void* x, const float* xs, const void* y, const float* ys, void* out,
+                                       const int32_t* tokens, int G, int M, int N, int64_t Ktot, int num_cu,
+                                       int32_t* queue) {
+  GemmParams p = zero_params();
+  p.A = x; p.B = y; p.C = out; p.sizes = tokens; p.sizes_i64 = 0; p.G = G;
+  p.scale_m = xs; p.scale_n = ys; p.scale_m_sg = M;
+  p.mode = MODE_KG_COUNT; p.m_total = M; p.k_total = Ktot; p.N = N; p.K = 0;
+  p.a_sm = Ktot; p.a_sk = 1; p.b_sg = 0; p.b_sn = Ktot; p.b_sk = 1; p.c_sg = (int64_t)M * N;
+  p.grid_limit = num_cu;
+  p.queue = queue;
+  return p;
+}
+
+static GemmParams params_fp8_block(const void* Aq, const float* sa, const void* Bq, const float* sb, void* C,
+                                   const void* sizes, int sizes_i64, const int32_t* row_start, int G, int64_t M, int N,
+                                   int K, int align, int sa_mn_major, int num_cu) {
+  GemmParams p = zero_params();
+  p.A = Aq; p.B = Bq; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
+  p.sa = sa; p.sb = sb;
+  const int kblocks = (K + 127) / 128;
+  if (sa_mn_major) { p.sa_rs = 1; p.sa_ks = M; } else { p.sa_rs = kblocks; p.sa_ks = 1; }
+  p.mode = MODE_MG_PAD; p.align = row_start ? 1 : align; p.row_start = row_start; p.m_total = M; p.N = N; p.K = K;
+  p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K; p.b_sn = K; p.b_sk = 1;
+  p.grid_limit = num_cu;
+  return p;
+}
+
 static int dispatch_16bit(const GemmParams& p, int dt, int layout, hipStream_t s) {
-  if (!g_force_generic && g_four_wave && w4_supported(p, dt, layout, g_four_wave == 2)) return launch_w4_16bit(p, dt, layout, s);
-  if (!g_force_generic && fast_supported(p, dt, layout)) return launch_fast_16bit(p, dt, layout, s);
+  const int force_generic = g_force_generic.load(), four_wave = g_four_wave.load();
+  if (!force_generic && four_wave && w4_supported(p, dt, layout, four_wave == 2)) return launch_w4_16bit(p, dt, layout, s);
+  if (!force_generic && fast_supported(p, dt, layout)) return launch_fast_16bit(p, dt, layout, s);
   return launch_generic_16bit(p, dt, layout, s);
 }
 
@@ -124,6 +218,56 @@ static int tile_order_host(const GemmParams& p, int grid, int split, int64_t* ou
   return n <= capacity ? 0 : set_error("tile order needs %lld rows, capacity %lld", (long long)n, (long long)capacity);
 }
 
+
+// Host-side walk of the shape-agnostic kernel's address arithmetic (generic_addr.hpp) over every tile of a launch:
+// lowest and highest element each operand is touched at.  out[op][0..1], op = A, B, C, scale_m, scale_n, sa, sb;
+// an operand that is never touched reports {INT64_MAX, -1}.
+template <bool A_KMAJOR, bool B_KMAJOR>
+static void generic_extents_host(const GemmParams& p, int epi, int64_t* out) {
+  SchedTable* t = new SchedTable;
+  for (int g = 0; g < p.G; ++g) sched_load_group(p, *t, g);
+  if (p.mode != MODE_KG) sched_prefix<kGenericBM>(p, *t);
+  if (generic_kmode(p)) sched_order_groups_serial(p, *t);
+  const int64_t total = sched_num_tiles<kGenericBM, kGenericBN>(p, *t);
+  for (int op = 0; op < 7; ++op) { out[2 * op] = INT64_MAX; out[2 * op + 1] = -1; }
+  auto touch = [&](int op, int64_t lo, int64_t hi) {
+    if (lo < out[2 * op]) out[2 * op] = lo;
+    if (hi > out[2 * op + 1]) out[2 * op + 1] = hi;
+  };
+  for (int64_t id = 0; id < total; ++id) {
+    const Tile tl = sched_tile<kGenericBM, kGenericBN>(p, *t, id);
+    const GenericTileIo io = generic_tile_io<A_KMAJOR>(p, tl);
+    const int64_t klen = tl.k1 - tl.k0;
+    const int kt_n = (int)((klen + kGenericBK - 1) / kGenericBK);
+    if (kt_n > 0 && io.a_lim > 0) {
+      if (A_KMAJOR) touch(0, io.a_elem + generic_elem_kmajor(0, p.a_sm, tl.k0), io.a_elem + generic_elem_kmajor(io.a_lim - 1, p.a_sm, tl.k1 - 1));
+      else touch(0, io.a_elem + generic_elem_mnmajor(tl.k0, p.a_sk, 0), io.a_elem + generic_elem_mnmajor(tl.k1 - 1, p.a_sk, io.a_lim - 1));
+    }
+    if (kt_n > 0 && io.b_lim > 0) {
+      if (B_KMAJOR) touch(1, io.b_elem + generic_elem_kmajor(0, p.b_sn, tl.k0), io.b_elem + generic_elem_kmajor(io.b_lim - 1, p.b_sn, tl.k1 - 1));
+      else touch(1, io.b_elem + generic_elem_mnmajor(tl.k0, p.b_sk, 0), io.b_elem + generic_elem_mnmajor(tl.k1 - 1, p.b_sk, io.b_lim - 1));
+    }
+    if (tl.rows > 0 && io.b_lim > 0) {
+      touch(2, io.c_elem + tl.n0, io.c_elem + (int64_t)(tl.rows - 1) * p.N + tl.n0 + io.b_lim - 1);
+      if (epi == 1) {
+        touch(3, generic_scale_m_index(p, tl, 0), generic_scale_m_index(p, tl, tl.rows - 1));
+        touch(4, generic_scale_n_index(p, tl, tl.n0), generic_scale_n_index(p, tl, tl.n0 + io.b_lim - 1));
+      }
+    }
+    if (epi == 2 && kt_n > 0) {
+      const int kb_last = generic_scale_block_of_slab(kt_n - 1);
+      touch(6, generic_sb_index(p, tl, 0), generic_sb_index(p, tl, kb_last));
+      if (tl.rows > 0) {
+        for (int kb = 0; kb <= kb_last; kb += (kb_last > 0 ? kb_last : 1)) {
+          touch(5, generic_sa_index(p, tl, 0, kb), generic_sa_index(p, tl, 0, kb));
+          touch(5, generic_sa_index(p, tl, tl.rows - 1, kb), generic_sa_index(p, tl, tl.rows - 1, kb));
+        }
+      }
+    }
+  }
+  delete t;
+}
+
 extern "C" {
 
 int tgg_m_grouped_gemm(const void* A, const void* B, void* C, const void* sizes, int sizes_i64, int G, int64_t M,
@@ -133,13 +277,7 @@ int tgg_m_grouped_gemm(const void* A, const void* B, void* C, const void* sizes,
   if (dtype != TGG_BF16 && dtype != TGG_F16) return set_error("data type code %d not supported", dtype);
   if ((K & 7) || (N & 7)) return set_error("N and K must be multiples of 8 (16-byte rows), got N=%d K=%d", N, K);
   if (M == 0) return 0;
-  GemmParams p = zero_params();
-  p.A = A; p.B = B; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
-  p.mode = MODE_MG; p.m_total = M; p.N = N; p.K = K;
-  p.a_sm = K; p.a_sk = 1;
-  p.b_sg = (int64_t)N * K;
-  if (trans_b) { p.b_sn = K; p.b_sk = 1; } else { p.b_sn = 1; p.b_sk = N; }
-  p.grid_limit = num_cu;
+  const GemmParams p = params_m_grouped(A, B, C, sizes, sizes_i64, G, M, N, K, trans_b, num_cu);
   return dispatch_16bit(p, dtype, trans_b ? 0 : 1, (hipStream_t)stream);
 }
 
@@ -153,13 +291,7 @@ int tgg_m_grouped_gemm_fp8_out(const void* A, const void* B, void* codes, float*
   if (fmt != DT_E4M3 && fmt != DT_E5M2) return set_error("unsupported fp8 format code %d", fmt);
   if ((K & 7) || (N & 127)) return set_error("K must be a multiple of 8 and N of 128, got N=%d K=%d", N, K);
   if (M == 0) return 0;
-  GemmParams p = zero_params();
-  p.A = A; p.B = B; p.C = codes; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
-  p.mode = MODE_MG; p.m_total = M; p.N = N; p.K = K;
-  p.a_sm = K; p.a_sk = 1;
-  p.b_sg = (int64_t)N * K;
-  if (trans_b) { p.b_sn = K; p.b_sk = 1; } else { p.b_sn = 1; p.b_sk = N; }
-  p.grid_limit = num_cu;
+  GemmParams p = params_m_grouped(A, B, codes, sizes, sizes_i64, G, M, N, K, trans_b, num_cu);
   p.q_scales = scales;
   p.q_fmt = fmt;
   if (scales_mn_major) { p.q_rs = 1; p.q_bs = M; } else { p.q_rs = N / 128; p.q_bs = 1; }
@@ -178,11 +310,7 @@ int tgg_m_grouped_gemm_padded(const void* A, const void* B, void* C, const void*
   if (dtype != TGG_BF16 && dtype != TGG_F16) return set_error("data type code %d not supported", dtype);
   if ((K & 7) || (N & 7)) return set_error("N and K must be multiples of 8 (16-byte rows), got N=%d K=%d", N, K);
   if (M == 0) return 0;
-  GemmParams p = zero_params();
-  p.A = A; p.B = B; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
-  p.mode = MODE_MG_PAD; p.align = align; p.m_total = M; p.N = N; p.K = K;
-  p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K; p.b_sn = K; p.b_sk = 1;
-  p.grid_limit = num_cu;
+  const GemmParams p = params_padded(A, B, C, sizes, sizes_i64, nullptr, G, M, N, K, align, num_cu);
   return dispatch_16bit(p, dtype, 0, (hipStream_t)stream);
 }
 
@@ -196,11 +324,7 @@ int tgg_m_grouped_gemm_placed(const void* A, const void* B, void* C, const void*
   if (dtype != TGG_BF16 && dtype != TGG_F16) return set_error("data type code %d not supported", dtype);
   if ((K & 7) || (N & 7)) return set_error("N and K must be multiples of 8 (16-byte rows), got N=%d K=%d", N, K);
   if (M == 0) return 0;
-  GemmParams p = zero_params();
-  p.A = A; p.B = B; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
-  p.mode = MODE_MG_PAD; p.align = 1; p.row_start = row_start; p.m_total = M; p.N = N; p.K = K;
-  p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K; p.b_sn = K; p.b_sk = 1;
-  p.grid_limit = num_cu;
+  const GemmParams p = params_padded(A, B, C, sizes, sizes_i64, row_start, G, M, N, K, 1, num_cu);
   return dispatch_16bit(p, dtype, 0, (hipStream_t)stream);
 }
 
@@ -212,12 +336,7 @@ int tgg_m_grouped_gemm_masked(const void* A, const void* B, void* C, const void*
   if (dtype != TGG_BF16 && dtype != TGG_F16) return set_error("data type code %d not supported", dtype);
   if ((K & 7) || (N & 7)) return set_error("N and K must be multiples of 8 (16-byte rows), got N=%d K=%d", N, K);
   if (M == 0 || m_stride == 0) return 0;
-  GemmParams p = zero_params();
-  p.A = A; p.B = B; p.C = C; p.sizes = masked_m; p.sizes_i64 = masked_i64; p.G = G;
-  p.mode = MODE_MASKED; p.m_stride = m_stride; p.m_total = M; p.N = N; p.K = K;
-  p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K;
-  if (trans_b) { p.b_sn = K; p.b_sk = 1; } else { p.b_sn = 1; p.b_sk = N; }
-  p.grid_limit = num_cu;
+  const GemmParams p = params_masked(A, B, C, masked_m, masked_i64, G, m_stride, M, N, K, trans_b, num_cu);
   return dispatch_16bit(p, dtype, trans_b ? 0 : 1, (hipStream_t)stream);
 }
 
@@ -233,12 +352,7 @@ int tgg_k_grouped_gemm_queued(const void* A, const void* B, void* C, const int32
   if (Mdim < 1 || Ktot < 0) return set_error("bad Mdim=%d or Ktot=%lld", Mdim, (long long)Ktot);
   if (dtype != TGG_BF16 && dtype != TGG_F16) return set_error("data type code %d not supported", dtype);
   if ((Mdim & 7) || (N & 7)) return set_error("Mdim and N must be multiples of 8 (16-byte rows), got %d, %d", Mdim, N);
-  GemmParams p = zero_params();
-  p.A = A; p.B = B; p.C = C; p.k_start = start; p.k_end = end; p.G = G;
-  p.mode = MODE_KG; p.m_total = Mdim; p.k_total = Ktot; p.N = N; p.K = 0;
-  p.a_sm = 1; p.a_sk = Mdim; p.b_sg = 0; p.b_sn = 1; p.b_sk = N; p.c_sg = (int64_t)Mdim * N;
-  p.grid_limit = num_cu;
-  p.queue = queue;
+  const GemmParams p = params_k_grouped(A, B, C, start, end, G, Mdim, N, Ktot, num_cu, queue);
   return dispatch_16bit(p, dtype, 2, (hipStream_t)stream);
 }
 
@@ -253,13 +367,8 @@ int tgg_m_grouped_gemm_fp8_channel(const void* Aq, const float* a_scale, const v
   if (!is_fp8(fmt_a) || !is_fp8(fmt_b)) return set_error("fp8 format codes must be E4M3 or E5M2");
   if (K & 15) return set_error("K must be a multiple of 16 for fp8 operands, got %d", K);
   if (M == 0) return 0;
-  GemmParams p = zero_params();
-  p.A = Aq; p.B = Bq; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
-  p.scale_m = a_scale; p.scale_n = b_scale;
-  p.mode = MODE_MG; p.m_total = M; p.N = N; p.K = K;
-  p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K; p.b_sn = K; p.b_sk = 1;
-  p.grid_limit = num_cu;
-  if (!g_force_generic && fast_fp8_supported(p, false)) return launch_fast_fp8_channel(p, fmt_a, fmt_b, out_dtype, (hipStream_t)stream);
+  const GemmParams p = params_fp8_channel(Aq, a_scale, Bq, b_scale, C, sizes, sizes_i64, G, M, N, K, num_cu);
+  if (!g_force_generic.load() && fast_fp8_supported(p, false)) return launch_fast_fp8_channel(p, fmt_a, fmt_b, out_dtype, (hipStream_t)stream);
   return launch_generic_fp8_channel(p, fmt_a, fmt_b, out_dtype, (hipStream_t)stream);
 }
 
@@ -277,19 +386,13 @@ int tgg_k_grouped_gemm_fp8_channel_queued(const void* x, const float* xs, const 
   if (M < 1 || Ktot < 0) return set_error("bad M=%d or Ktot=%lld", M, (long long)Ktot);
   if (!is_fp8(fmt_a) || !is_fp8(fmt_b)) return set_error("fp8 format codes must be E4M3 or E5M2");
   if (Ktot & 15) return set_error("Ktot must be a multiple of 16 for fp8 operands, got %lld", (long long)Ktot);
-  GemmParams p = zero_params();
-  p.A = x; p.B = y; p.C = out; p.sizes = tokens; p.sizes_i64 = 0; p.G = G;
-  p.scale_m = xs; p.scale_n = ys; p.scale_m_sg = M;
-  p.mode = MODE_KG_COUNT; p.m_total = M; p.k_total = Ktot; p.N = N; p.K = 0;
-  p.a_sm = Ktot; p.a_sk = 1; p.b_sg = 0; p.b_sn = Ktot; p.b_sk = 1; p.c_sg = (int64_t)M * N;
-  p.grid_limit = num_cu;
-  p.queue = queue;
-  if (!g_force_generic && fast_fp8_supported(p, false)) {
+  GemmParams p = params_fp8_k_channel(x, xs, y, ys, out, tokens, G, M, N, Ktot, num_cu, queue);
+  if (!g_force_generic.load() && fast_fp8_supported(p, false)) {
     // The tuned kernel needs every token count to be a multiple of 16 and only the device knows the counts: both
     // kernels are enqueued, each reads the counts first and exactly one of them runs (the other returns at once).
     p.kg_gate = 1;
     if (int e = launch_fast_fp8_channel(p, fmt_a, fmt_b, TGG_BF16, (hipStream_t)stream)) return e;
-    if (!g_kg_second_launch) return 0;
+    if (!g_kg_second_launch.load()) return 0;
     p.kg_gate = 2;
   }
   return launch_generic_fp8_channel(p, fmt_a, fmt_b, TGG_BF16, (hipStream_t)stream);
@@ -305,15 +408,9 @@ static int fp8_block_impl(const void* Aq, const float* sa, const void* Bq, const
   if (!row_start && (align < 1 || (align & 127))) return set_error("alignment must be a positive multiple of 128, got %d", align);
   if (K & 15) return set_error("K must be a multiple of 16 for fp8 operands, got %d", K);
   if (M == 0) return 0;
-  GemmParams p = zero_params();
-  p.A = Aq; p.B = Bq; p.C = C; p.sizes = sizes; p.sizes_i64 = sizes_i64; p.G = G;
-  p.sa = sa; p.sb = sb;
+  const GemmParams p = params_fp8_block(Aq, sa, Bq, sb, C, sizes, sizes_i64, row_start, G, M, N, K, align, sa_mn_major, num_cu);
   const int kblocks = (K + 127) / 128;
-  if (sa_mn_major) { p.sa_rs = 1; p.sa_ks = M; } else { p.sa_rs = kblocks; p.sa_ks = 1; }
-  p.mode = MODE_MG_PAD; p.align = row_start ? 1 : align; p.row_start = row_start; p.m_total = M; p.N = N; p.K = K;
-  p.a_sm = K; p.a_sk = 1; p.b_sg = (int64_t)N * K; p.b_sn = K; p.b_sk = 1;
-  p.grid_limit = num_cu;
-  if (!g_force_generic && sa_mn_major && kblocks <= 64 && fast_fp8_supported(p, true))
+  if (!g_force_generic.load() && sa_mn_major && kblocks <= 64 && fast_fp8_supported(p, true))
     return launch_fast_fp8_block(p, (hipStream_t)stream);
   return launch_generic_fp8_block(p, (hipStream_t)stream);
 }
@@ -472,6 +569,61 @@ int tgg_debug_tile_order(const int64_t* sizes, int G, int mode, int64_t m_total,
   if (tile == 256) return tile_order_host<256, 256>(p, grid, split, out, capacity, num_tiles);
   if (tile == 128) return tile_order_host<128, 128>(p, grid, split, out, capacity, num_tiles);
   return set_error("tile must be 256 (tuned kernels) or 128 (shape-agnostic kernel)");
+}
+
+int tgg_debug_generic_extents(int kind, const int64_t* sizes, const int32_t* row_start, int G, int64_t M, int64_t aux,
+                              int N, int K, int64_t* out) {
+  if (!sizes || !out) return set_error("null pointer");
+  if (G < 1 || G > TGG_MAX_GROUPS) return set_error("G=%d outside [1, %d]", G, TGG_MAX_GROUPS);
+  if (N < 1 || M < 0 || K < 0) return set_error("bad M / N / K");
+  // Non-null dummies: the walk computes offsets, it dereferences only `sizes`, `row_start` and the k ranges.
+  static char dummy;
+  const void* D = &dummy;
+  std::vector<int32_t> counts(sizes, sizes + G), ks(G), ke(G);
+  switch (kind) {
+    case 0: case 1: {  // tgg_m_grouped_gemm, trans_b = 1 / 0
+      const GemmParams p = params_m_grouped(D, D, &dummy, sizes, 1, G, M, N, K, kind == 0, -1);
+      if (kind == 0) generic_extents_host<true, true>(p, 0, out); else generic_extents_host<true, false>(p, 0, out);
+      return 0;
+    }
+    case 2: {  // tgg_m_grouped_gemm_masked, aux = m_stride
+      const GemmParams p = params_masked(D, D, &dummy, sizes, 1, G, aux, M, N, K, 1, -1);
+      generic_extents_host<true, true>(p, 0, out);
+      return 0;
+    }
+    case 3: case 4: {  // tgg_m_grouped_gemm_padded (aux = align) / _placed (row_start)
+      if (kind == 4 && !row_start) return set_error("placed launches need row_start");
+      if (kind == 3 && aux < 1) return set_error("alignment must be positive");
+      const GemmParams p = params_padded(D, D, &dummy, sizes, 1, kind == 4 ? row_start : nullptr, G, M, N, K, (int)aux, -1);
+      generic_extents_host<true, true>(p, 0, out);
+      return 0;
+    }
+    case 5: {  // tgg_k_grouped_gemm: sizes = token counts, M = Mdim, aux = Ktot
+      int64_t at = 0;
+      for (int g = 0; g < G; ++g) { ks[g] = (int32_t)at; at += sizes[g] < 0 ? 0 : sizes[g]; ke[g] = (int32_t)at; }
+      const GemmParams p = params_k_grouped(D, D, &dummy, ks.data(), ke.data(), G, (int)M, N, aux, -1, nullptr);
+      generic_extents_host<false, false>(p, 0, out);
+      return 0;
+    }
+    case 6: {  // tgg_m_grouped_gemm_fp8_channel
+      const GemmParams p = params_fp8_channel(D, (const float*)D, D, (const float*)D, &dummy, sizes, 1, G, M, N, K, -1);
+      generic_extents_host<true, true>(p, 1, out);
+      return 0;
+    }
+    case 7: {  // tgg_k_grouped_gemm_fp8_channel: sizes = token counts (int32 in the ABI), M rows of x, aux = Ktot
+      const GemmParams p = params_fp8_k_channel(D, (const float*)D, D, (const float*)D, &dummy, counts.data(), G, (int)M, N, aux, -1, nullptr);
+      generic_extents_host<true, true>(p, 1, out);
+      return 0;
+    }
+    case 8: case 9: case 10: {  // tgg_m_grouped_gemm_fp8_block: aux = align; 8 = sa [M, KB], 9 = sa [KB, M], 10 = placed ([KB, M])
+      if (kind == 10 && !row_start) return set_error("placed launches need row_start");
+      const GemmParams p = params_fp8_block(D, (const float*)D, D, (const float*)D, &dummy, sizes, 1,
+                                            kind == 10 ? row_start : nullptr, G, M, N, K, (int)aux, kind != 8, -1);
+      generic_extents_host<true, true>(p, 2, out);
+      return 0;
+    }
+  }
+  return set_error("unknown kind %d", kind);
 }
 
 int tgg_debug_queue_order(int grid, int draws, int32_t* out) {

@@ -32,6 +32,7 @@
 //     leave as 16-byte stores that cover whole row segments of the wave's columns.
 #include "fast_common.hpp"
 #include "launch.hpp"
+#include <atomic>
 #include <type_traits>
 
 namespace tgg {
@@ -684,6 +685,7 @@ TGG_DEV void gemm_fast_body(const GemmParams& p) {
       }
     }
   }
+  if (LAYOUT == LAYOUT_TN && queued && threadIdx.x == 0) sched_queue_finish(p.queue);
   wait_vmcnt<0>();  // the trailing zero-length copies still write LDS: let them finish before the wave ends
 }
 
@@ -773,7 +775,7 @@ int launch_auto(const GemmParams& p, hipStream_t s) {
   return launch_kernel(gemm_fast_auto_kernel<CW, CN, CS, DT, LAYOUT>, CW::SMEM_BYTES, CW::THREADS, attr_flag(attr_set), p, s, "gemm_fast");
 }
 
-int g_variant = 0;
+std::atomic<int> g_variant{0};
 
 template <int DT, int LAYOUT>
 int launch_variant(const GemmParams& p, hipStream_t s) {
@@ -781,7 +783,7 @@ int launch_variant(const GemmParams& p, hipStream_t s) {
   typedef FastCfg<256, 128, 2, 4> Narrow;
   typedef FastCfg<128, 256, 2, 4, 3> Stream;
   typedef typename std::conditional<LAYOUT == LAYOUT_TN, void, Stream>::type StreamOrNone;
-  switch (g_variant) {
+  switch (g_variant.load()) {
     default:
     case 0: return launch_auto<Wide, Narrow, StreamOrNone, DT, LAYOUT>(p, s);
     case 1: return launch_cfg<Narrow, DT, LAYOUT, false>(p, s);

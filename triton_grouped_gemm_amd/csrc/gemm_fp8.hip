@@ -17,6 +17,7 @@
 //                the epilogue; used M-grouped and K-grouped (per-group token range along K).
 #include "fast_common.hpp"
 #include "launch.hpp"
+#include <atomic>
 
 namespace tgg {
 
@@ -573,6 +574,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
       }
     }
   }
+  if (KGROUP && queued && threadIdx.x == 0) sched_queue_finish(p.queue);
   wait_vmcnt<0>();  // the trailing zero-length copies still write LDS: let them finish before the wave ends
 }
 
@@ -646,19 +648,20 @@ typedef Fp8Cfg<256, 256, 2, 4> Fp8Wide;
 typedef Fp8Cfg<256, 128, 2, 4> Fp8Narrow;
 typedef Fp8Cfg<128, 256, 2, 4, 3> Fp8Stream;
 
-int g_fp8_variant = 0;  // 0: chosen on the device (M-grouped), 1: narrow, 2: wide, 4: weight-streaming configuration
+std::atomic<int> g_fp8_variant{0};  // 0: chosen on the device (M-grouped), 1: narrow, 2: wide, 4: weight-streaming configuration
 
 // M-grouped launches choose the tile width on the device; K-grouped ones (tile count known to the host, tile cost
 // set by the group's token count) use the wide tiles.
 template <int FA, int FB, int EPI, int OUT, bool KGROUP>
 int launch_fp8_cfg(const GemmParams& p, hipStream_t s) {
   static bool attr_auto[64] = {false}, attr_wide[64] = {false}, attr_narrow[64] = {false}, attr_stream[64] = {false};
+  const int variant = g_fp8_variant.load();
   if constexpr (!KGROUP) {
-    if (g_fp8_variant == 0)
+    if (variant == 0)
       return launch_fp8_kernel(gemm_fp8_auto_kernel<Fp8Wide, Fp8Narrow, Fp8Stream, FA, FB, EPI, OUT>, Fp8Wide::SMEM_BYTES, Fp8Wide::THREADS, attr_auto, p, s);
-    if (g_fp8_variant == 4)
+    if (variant == 4)
       return launch_fp8_kernel(gemm_fp8_kernel<Fp8Stream, FA, FB, EPI, OUT, false>, Fp8Stream::SMEM_BYTES, Fp8Stream::THREADS, attr_stream, p, s);
-    if (g_fp8_variant == 1)
+    if (variant == 1)
       return launch_fp8_kernel(gemm_fp8_kernel<Fp8Narrow, FA, FB, EPI, OUT, false>, Fp8Narrow::SMEM_BYTES, Fp8Narrow::THREADS, attr_narrow, p, s);
   }
   return launch_fp8_kernel(gemm_fp8_kernel<Fp8Wide, FA, FB, EPI, OUT, KGROUP>, Fp8Wide::SMEM_BYTES, Fp8Wide::THREADS, attr_wide, p, s);

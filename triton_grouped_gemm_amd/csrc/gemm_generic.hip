@@ -11,13 +11,14 @@
 // gemm_fast.hip take over for the aligned shapes.
 #include "common.hpp"
 #include "sched.hpp"
+#include "generic_addr.hpp"
 #include "launch.hpp"
 
 namespace tgg {
 
 namespace {
 
-constexpr int GBM = 128, GBN = 128, GBK = 32, GTHREADS = 256;
+constexpr int GBM = kGenericBM, GBN = kGenericBN, GBK = kGenericBK, GTHREADS = 256;
 
 template <int DT> struct ElemSize { static constexpr int v = (DT <= DT_F16) ? 2 : 1; };
 
@@ -83,7 +84,7 @@ template <int DT, bool KMAJOR> struct Stager {
         const int row = idx / VPR;
         const int64_t kk = k + (idx % VPR) * VEC;
         if (row < lim_mn && kk < k_end) {
-          const char* src = base + ((int64_t)row * s_row + kk) * ES;
+          const char* src = base + generic_elem_kmajor(row, s_row, kk) * ES;
           if (kk + VEC <= k_end) val = *(const i32x4_t*)src;
           else val = load_partial(src, (int)(k_end - kk) * ES);
         }
@@ -93,7 +94,7 @@ template <int DT, bool KMAJOR> struct Stager {
         const int mn = (idx % VPR) * VEC;
         const int64_t kk = k + krow;
         if (kk < k_end && mn < lim_mn) {
-          const char* src = base + (kk * s_k + mn) * ES;
+          const char* src = base + generic_elem_mnmajor(kk, s_k, mn) * ES;
           if (mn + VEC <= lim_mn) val = *(const i32x4_t*)src;
           else val = load_partial(src, (lim_mn - mn) * ES);
         }
@@ -152,18 +153,12 @@ __global__ __launch_bounds__(GTHREADS) void gemm_generic_kernel(const GemmParams
   const TileWalk walk = sched_walk(num_tiles, !kmode);
   for (int64_t tile_id = walk.first; tile_id < walk.end; tile_id += walk.stride) {
     const Tile t = sched_tile<GBM, GBN>(p, sm.sched, tile_id);
-    // operand bases for this tile at k = 0
-    const char* a_base;
-    int a_lim;
-    if (kmode) {  // rows of the tile are columns m of A[Ktot, Mdim]
-      a_base = (const char*)p.A + (A_KMAJOR ? t.row0 * p.a_sm : t.row0) * ESA;
-      a_lim = t.rows;
-    } else {
-      a_base = (const char*)p.A + t.row0 * p.a_sm * ESA;
-      a_lim = t.rows;
-    }
-    const char* b_base = (const char*)p.B + ((int64_t)t.g * p.b_sg + (int64_t)t.n0 * p.b_sn) * ESB;
-    const int b_lim = (p.N - t.n0) < GBN ? (p.N - t.n0) : GBN;
+    // operand bases for this tile at k = 0 (generic_addr.hpp)
+    const GenericTileIo io = generic_tile_io<A_KMAJOR>(p, t);
+    const char* a_base = (const char*)p.A + io.a_elem * ESA;
+    const int a_lim = io.a_lim;
+    const char* b_base = (const char*)p.B + io.b_elem * ESB;
+    const int b_lim = io.b_lim;
 
     f32x16_t acc[2][2];
     f32x16_t part[2][2];
@@ -211,14 +206,12 @@ __global__ __launch_bounds__(GTHREADS) void gemm_generic_kernel(const GemmParams
         // every 128 of K (or at the end) fold the partial sums in with their block scales
         const int64_t kpos = (int64_t)(kt + 1) * GBK;
         if ((kpos & 127) == 0 || kt + 1 == kt_n) {
-          const int kb = (int)((kpos - 1) >> 7);
-          const int kblocks = (p.K + 127) >> 7;
-          const int nblocks = (p.N + 127) >> 7;
-          const float sbv = p.sb[((int64_t)t.g * nblocks + (t.n0 >> 7)) * kblocks + kb];
+          const int kb = generic_scale_block_of_slab(kt);
+          const float sbv = p.sb[generic_sb_index(p, t, kb)];
 #pragma unroll
           for (int i = 0; i < 2; ++i) {
             const int m = wm + i * 32 + l32;
-            const float s = (m < t.rows) ? p.sa[(t.row0 + m) * p.sa_rs + kb * p.sa_ks] * sbv : 0.f;
+            const float s = (m < t.rows) ? p.sa[generic_sa_index(p, t, m, kb)] * sbv : 0.f;
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -237,14 +230,14 @@ __global__ __launch_bounds__(GTHREADS) void gemm_generic_kernel(const GemmParams
     }
 
     // epilogue: lane owns row m, columns n = wn + j*32 + 8q + 4*lh + (0..3)
-    char* c_base = (char*)p.C + (kmode ? ((int64_t)t.g * p.c_sg + t.row0 * p.N) : t.row0 * (int64_t)p.N) * 2;
+    char* c_base = (char*)p.C + io.c_elem * 2;
     const bool vec_ok = (p.N & 3) == 0;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int m = wm + i * 32 + l32;
       if (m >= t.rows) continue;
       float rs = 1.f;
-      if (EPI == EPI_CHANNEL) rs = kmode ? p.scale_m[(int64_t)t.g * p.scale_m_sg + t.row0 + m] : p.scale_m[t.row0 + m];
+      if (EPI == EPI_CHANNEL) rs = p.scale_m[generic_scale_m_index(p, t, m)];
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -255,7 +248,7 @@ __global__ __launch_bounds__(GTHREADS) void gemm_generic_kernel(const GemmParams
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             v[e] = acc[i][j][q * 4 + e];
-            if (EPI == EPI_CHANNEL) v[e] = (n + e < p.N) ? v[e] * rs * p.scale_n[(int64_t)t.g * p.N + n + e] : 0.f;
+            if (EPI == EPI_CHANNEL) v[e] = (n + e < p.N) ? v[e] * rs * p.scale_n[generic_scale_n_index(p, t, n + e)] : 0.f;
           }
           char* dst = c_base + ((int64_t)m * p.N + n) * 2;
           if (vec_ok) {

@@ -70,7 +70,7 @@ TGG_HD void sched_prefix(const GemmParams& p, Table& t) {
       row += (p.mode == MODE_MG_PAD) ? ((sz + p.align - 1) / p.align) * p.align : sz;
     }
     const int64_t limit = (p.mode == MODE_KG_COUNT) ? p.k_total : p.m_total;
-    if (start >= limit) sz = 0;  // never touch rows (or k) past the end of the operands
+    if (start < 0 || start >= limit) sz = 0;  // never touch rows (or k) outside the operands (a negative start can only come from row_start)
     else if (start + sz > limit) sz = limit - start;
     t.row0[g] = start;
     t.rows[g] = (int32_t)sz;
@@ -173,7 +173,7 @@ TGG_DEV int32_t sched_init(const GemmParams& p, Table& t) {
     if (p.mode == MODE_MG_PAD && p.row_start && live) start = (int64_t)p.row_start[g];
   }
   const int64_t limit = (p.mode == MODE_KG_COUNT) ? p.k_total : p.m_total;
-  if (start >= limit) sz = 0;  // never touch rows (or k) past the end of the operands
+  if (start < 0 || start >= limit) sz = 0;  // never touch rows (or k) outside the operands (a negative start can only come from row_start)
   else if (start + sz > limit) sz = limit - start;
   constexpr int HALF = BM / 2;
   int64_t total;
@@ -394,6 +394,16 @@ TGG_DEV int sched_draw_tile(int32_t* queue, int total, int& victim) {
     ++victim;
   }
   return total;
+}
+
+// End of a queued launch: every workgroup reports here once it has drawn its last id (the draw that found all eight
+// counters exhausted has returned by then), and the workgroup that reports last puts the nine words back to zero, so
+// that the next launch on the same stream finds the queue as this one found it.  Thread 0 of each workgroup calls it.
+constexpr int kQueueDoneWord = 8;
+TGG_DEV void sched_queue_finish(int32_t* queue) {
+  if (atomicAdd(queue + kQueueDoneWord, 1) == (int)gridDim.x - 1) {
+    for (int i = 0; i <= kQueueDoneWord; ++i) atomicExch(queue + i, 0);
+  }
 }
 
 }  // namespace tgg

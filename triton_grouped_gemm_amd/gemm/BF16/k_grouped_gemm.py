@@ -47,9 +47,13 @@ def _check_k_grouped_gemm_inputs(A: Tensor, B: Tensor, size_per_group: Tensor, t
 
 def k_grouped_gemm(A: Tensor, B: Tensor, size_per_group: Tensor, group_start: Optional[Tensor] = None,
                    group_end: Optional[Tensor] = None, trans_b: bool = False, numSM: int = -1,
-                   use_fixed_sm90_config: bool = True) -> Tensor:
+                   use_fixed_sm90_config: bool = True, *, queue: Optional[Tensor] = None) -> Tensor:
     """A ``[K_TOTAL, M_DIM]``, B ``[K_TOTAL, N_DIM]`` -> C ``[G, M_DIM, N_DIM]`` (fp32 accumulation over
-    the whole segment, one rounding to the input dtype)."""
+    the whole segment, one rounding to the input dtype).
+
+    ``queue`` (not in the reference): the kernel's tile counters, ``_native.QUEUE_WORDS`` zeroed int32 on A's device
+    that the caller owns -- for callers that must not allocate inside the call (graph capture); the kernel hands them
+    back zeroed.  By default the library keeps one such tensor per device and stream."""
     K_TOTAL, M_DIM, N_DIM, num_groups = _check_k_grouped_gemm_inputs(A, B, size_per_group, trans_b)
     assert 1 <= num_groups <= _native.MAX_GROUPS, f"between 1 and {_native.MAX_GROUPS} groups are supported"
     C = A.new_empty(num_groups, M_DIM, N_DIM)
@@ -59,7 +63,7 @@ def k_grouped_gemm(A: Tensor, B: Tensor, size_per_group: Tensor, group_start: Op
     group_start = group_start.to(device=A.device, dtype=torch.int32).contiguous()
     group_end = group_end.to(device=A.device, dtype=torch.int32).contiguous()
     # tile-id counter of the kernel's work queue (a tile costs what its group has tokens; see include/tgg_amd.h)
-    queue = torch.zeros(_native.QUEUE_WORDS, dtype=torch.int32, device=A.device)
+    queue = _native.work_queue(A.device, queue)
     _native.call("tgg_k_grouped_gemm_queued", A.data_ptr(), B.data_ptr(), C.data_ptr(), group_start.data_ptr(),
                  group_end.data_ptr(), num_groups, M_DIM, N_DIM, K_TOTAL, _dtype_code(A.dtype), int(numSM),
                  queue.data_ptr(), _native.stream_of(A))

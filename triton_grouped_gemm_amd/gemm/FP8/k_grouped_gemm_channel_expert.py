@@ -7,6 +7,8 @@ tokens to a multiple of 128 with zeros, as the reference requires).
 """
 from __future__ import annotations
 
+from typing import Optional
+
 import torch
 from torch import Tensor
 
@@ -27,9 +29,11 @@ def _expert_major(scale: Tensor, rows: int, groups: int) -> Tensor:
 
 
 def matmul(x_fp8: Tensor, x_scale: Tensor, y_fp8: Tensor, y_scale: Tensor, tokens_per_expert: Tensor,
-           M: int, N: int, K: int, num_groups: int, dtype_a: int = 1, dtype_b: int = 1) -> Tensor:
+           M: int, N: int, K: int, num_groups: int, dtype_a: int = 1, dtype_b: int = 1, *,
+           queue: Optional[Tensor] = None) -> Tensor:
     """x ``[M, K]``, y ``[N, K]`` fp8 with the token dimension contiguous; dtype codes 1 = e4m3fn,
-    anything else = e5m2 (reference :83-84).  Returns ``[num_groups, M, N]`` bf16."""
+    anything else = e5m2 (reference :83-84).  Returns ``[num_groups, M, N]`` bf16.  ``queue`` (not in the
+    reference): caller-owned tile counters, see ``k_grouped_gemm``."""
     assert x_fp8.dim() == 2 and tuple(x_fp8.shape) == (M, K), "x_fp8 must be [M, K]"
     assert y_fp8.dim() == 2 and tuple(y_fp8.shape) == (N, K), "y_fp8 must be [N, K]"
     assert x_fp8.element_size() == 1 and y_fp8.element_size() == 1, "x_fp8 and y_fp8 must hold 8-bit codes"
@@ -42,7 +46,7 @@ def matmul(x_fp8: Tensor, x_scale: Tensor, y_fp8: Tensor, y_scale: Tensor, token
     tokens = tokens_per_expert.to(device=x_fp8.device, dtype=torch.int32).contiguous()
     output = torch.empty((num_groups, M, N), dtype=torch.bfloat16, device=x_fp8.device)
     # tile-id counter of the kernel's work queue (a tile costs what its group has tokens; see include/tgg_amd.h)
-    queue = torch.zeros(_native.QUEUE_WORDS, dtype=torch.int32, device=x_fp8.device)
+    queue = _native.work_queue(x_fp8.device, queue)
     _native.call("tgg_k_grouped_gemm_fp8_channel_queued", x_fp8.data_ptr(), xs.data_ptr(), y_fp8.data_ptr(),
                  ys.data_ptr(), output.data_ptr(), tokens.data_ptr(), num_groups, M, N, K,
                  _FMT.get(int(dtype_a), _native.E5M2), _FMT.get(int(dtype_b), _native.E5M2), -1, queue.data_ptr(),

@@ -69,8 +69,11 @@ def sizes_from_layout(grouped_layout: torch.Tensor, num_groups: int, block_m: in
         prev = torch.cat([lay.new_zeros(1), lay[:-1]])
         starts = (prev + (block_m - 1)) // block_m * block_m
         return (lay - starts).to(torch.int32)
+    # slot 0 collects the padding rows (-1) and, so that no id can index outside the table, every id that names no
+    # expert of b (below -1 or >= num_groups): those rows belong to no group and are not computed
+    slot = torch.where((lay >= 0) & (lay < num_groups), lay + 1, torch.zeros_like(lay))
     counts = torch.zeros(num_groups + 1, dtype=torch.int64, device=lay.device)
-    counts.scatter_add_(0, lay + 1, torch.ones_like(lay))
+    counts.scatter_add_(0, slot, torch.ones_like(lay))
     return counts[1:].to(torch.int32)
 
 
@@ -83,7 +86,9 @@ def placement_from_layout(grouped_layout: torch.Tensor, num_groups: int
     is None.  Some expert's rows in several regions: one entry per region (maximal run of rows with the same
     non-negative id) in row order, and expert ``[regions]`` (int64) names the expert of each, for the caller to
     gather the weights by.  Telling the two cases apart takes one read-back of two counters; while the current
-    stream is being captured it is left out and the first form is returned.  Reference contract:
+    stream is being captured it is left out and the first form is returned: a captured call therefore needs one
+    region per expert (several regions would be served as the single span from the expert's first row on), and ids
+    outside [-1, num_groups), which raise ValueError eagerly, are treated as padding there.  Reference contract:
     gemm/layout.py:73-97 builds such layouts in ascending expert order, gemm/deep_gemm_ops.py:24-100 forwards
     whatever the caller passes.
     """
@@ -96,9 +101,9 @@ def placement_from_layout(grouped_layout: torch.Tensor, num_groups: int
         seen = torch.zeros(num_groups + 1, dtype=torch.bool, device=dev)  # last slot: padding and ids out of range
         seen[torch.where((lay >= 0) & (lay < num_groups), lay, num_groups)] = True
         n_regions, n_experts, n_bad = torch.stack([(change & (lay >= 0)).sum(), seen[:num_groups].sum(),
-                                                   (lay >= num_groups).sum()]).tolist()
+                                                   ((lay >= num_groups) | (lay < -1)).sum()]).tolist()
         if n_bad:
-            raise ValueError(f"grouped_layout names experts beyond the {num_groups} that b holds")
+            raise ValueError(f"grouped_layout holds ids outside [-1, {num_groups}): b has {num_groups} experts and -1 marks padding")
         if n_regions > n_experts:
             if n_regions > _native.MAX_GROUPS_OTHER:
                 raise ValueError(f"grouped_layout has {n_regions} separate regions, at most {_native.MAX_GROUPS_OTHER} are supported")
@@ -106,10 +111,12 @@ def placement_from_layout(grouped_layout: torch.Tensor, num_groups: int
             lengths = torch.diff(starts, append=starts.new_tensor([m]))
             keep = lay[starts] >= 0
             return lengths[keep].to(torch.int32), starts[keep].to(torch.int32), lay[starts][keep]
+    # under capture nothing was checked: ids that name no expert go to the padding slot instead of indexing outside
+    slot = torch.where((lay >= 0) & (lay < num_groups), lay + 1, torch.zeros_like(lay))
     counts = torch.zeros(num_groups + 1, dtype=torch.int64, device=dev)
-    counts.scatter_add_(0, lay + 1, torch.ones_like(lay))
+    counts.scatter_add_(0, slot, torch.ones_like(lay))
     first = torch.full((num_groups + 1,), m, dtype=torch.int64, device=dev)
-    first.scatter_reduce_(0, lay + 1, torch.arange(m, dtype=torch.int64, device=dev), reduce="amin")
+    first.scatter_reduce_(0, slot, torch.arange(m, dtype=torch.int64, device=dev), reduce="amin")
     first = torch.where(counts > 0, first, torch.zeros_like(first))
     return counts[1:].to(torch.int32), first[1:].to(torch.int32), None
 
