@@ -156,6 +156,39 @@ def test_cast_recipes_match_torch_expressions():
     assert sz[0, 0] == np.float32(np.float32(1e-4) / np.float32(448.0)) and not cz.any()
 
 
+@pytest.mark.parametrize("shape", [(130, 200), (256, 384), (300, 520), (128, 8192)])
+def test_per_block_cast_matches_the_torch_expression_codes_and_scales(shape):
+    """quant_ref.per_block_cast_to_fp8 against the torch expression of the reference's per_block_cast_to_fp8
+    (gemm/FP8/m_grouped_gemm_channel_expert.py:237-245), evaluated by torch on the CPU: every code and every scale.
+    A division in place of torch's reciprocal-then-multiply for `448.0 / amax` changes codes and fails here."""
+    m, n = shape
+    x = _bf16_randn(shape, 60 + m, scale=2.0)
+    x[5, 7] = 0.0
+    if m > 256:
+        x[256:, 384:] *= 1e-3   # a ragged corner block of small values
+    xt = torch.from_numpy(x).to(torch.bfloat16)
+    x = xt.float().numpy()
+    codes, scales = quant_ref.per_block_cast_to_fp8(x)
+    mp, np_ = -(-m // 128) * 128, -(-n // 128) * 128
+    x_padded = torch.zeros((mp, np_), dtype=xt.dtype)
+    x_padded[:m, :n] = xt
+    x_view = x_padded.view(-1, 128, np_ // 128, 128)
+    x_amax = x_view.abs().float().amax(dim=(1, 3), keepdim=True).clamp(1e-4)
+    x_scaled = (x_view * (448.0 / x_amax)).to(torch.float8_e4m3fn)
+    ref_codes = x_scaled.view_as(x_padded)[:m, :n].contiguous().view(torch.uint8).numpy()
+    ref_scales = (x_amax / 448.0).view(x_view.size(0), x_view.size(2)).numpy()
+    assert codes.shape == (m, n) and scales.shape == ref_scales.shape
+    assert np.array_equal(codes, ref_codes)
+    assert np.array_equal(scales.view(np.uint32), ref_scales.view(np.uint32))
+    if shape != (128, 8192):
+        return
+    # the pin bites: with 64 blocks, one IEEE division instead of reciprocal * 448 changes hundreds of codes
+    amax = np.maximum(np.abs(np.pad(x, ((0, mp - m), (0, np_ - n)))).reshape(mp // 128, 128, np_ // 128, 128).max(axis=(1, 3), keepdims=True), np.float32(1e-4)).astype(np.float32)
+    wrong = (np.pad(x, ((0, mp - m), (0, np_ - n))).reshape(mp // 128, 128, np_ // 128, 128) * (np.float32(448.0) / amax)).astype(np.float32)
+    from oracle import fp8_soft
+    assert not np.array_equal(fp8_soft.encode_e4m3fn(wrong).reshape(mp, np_)[:m, :n], ref_codes)
+
+
 def test_row_and_expert_cast_recipes_match_torch_expressions():
     """per_row_cast_to_fp8 / per_expert_cast_to_fp8 against the torch expressions of the reference's
     per_channel_cast_to_fp8 and per_expert_cast_to_fp8 (gemm/FP8/m_grouped_gemm_channel_expert.py:224-234, :247-261):
