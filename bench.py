@@ -7,13 +7,24 @@ roofline fraction of the GEMM kernel (HIP-event timed on the launch stream) and,
 reference's per-group torch matmul timed on this box's host cores over a bounded sample of groups.
 
 With no flags the same run also times the FP8 block-scaled M-grouped configuration (the other half of the
-headline metric) and reports it under the "fp8" key of the line.
+headline metric, under the "fp8" key of the line, with its own CPU baseline) and the other configurations of the
+path, each with its roofline: "masked" (decode-style masked GEMM: the HBM roof binds, the MFMA figure sits beside
+it), "k_grouped" (weight gradient), "quant_trans128" (transposing 128x128 quantizer) and "quant_token128" (1x128
+activation quantizer).
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--uniform-groups] [--no-cpu-baseline]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--dtype bf16|fp16]
+                  [--uniform-groups | --random-groups [--unaligned-random-groups] [--group-align 64]]
+                  [--no-cpu-baseline] [--no-extras]
+  python bench.py --reference-cases [--only-model 30B|235B] [--groups 128] [--active 10] [--warmup 5] [--seed 2026]
+                  [--dtype bf16|fp16] [--random-groups ...] [--skip-check] [--skip-vendor] [--csv out.csv]
+      the sixteen cases of the reference's own benchmark main (gemm/BF16/m_grouped_gemm_TMA.py:474-493, :602-800),
+      with its flags, its group-size draws, its correctness gate and its CSV columns; prints its per-case lines.
 """
 from __future__ import annotations
 
 import argparse
+import csv
+import hashlib
 import json
 import os
 import sys
@@ -31,21 +42,57 @@ PEAK_HBM_GBS = 8000.0
 # (--pmc FETCH_SIZE and --pmc WRITE_SIZE, one counter per run, each scaled by what the counter reads for a
 # plain 1 GiB device copy: x2.0 and x1.0).  The runs and their figures are listed in profiles/hbm_traffic.txt.
 # FETCH_SIZE includes L2 fills served by the memory-side cache, so these are upper bounds on DRAM traffic.
+# Each figure belongs to the kernel sources it was measured with: name -> (GB, source set).  `roofline.traffic` is
+# printed only while the hash of that source set still equals the stamp below; after any change to those files it
+# is null until the counters are read again (python bench.py --print-traffic-stamps prints the current hashes).
 MEASURED_TRAFFIC_GB = {
-    "bf16_m_grouped_gateup_nt": 11.98,
-    "bf16_m_grouped_gateup_nn": 11.94,
-    "bf16_m_grouped_gateup_fp8_out": 10.69,
-    "bf16_m_grouped_down_nt": 5.38,
-    "bf16_m_grouped_down_nn": 5.42,
-    "bf16_masked_decode": 2.51,
-    "bf16_k_grouped_wgrad": 28.31,
-    "fp8_block_m_grouped": 29.07,
-    "fp8_channel_m_grouped": 27.73,
-    "fp8_channel_k_grouped": 18.05,
-    "quant_trans128": 8.12,
-    "moe_permute": 3.06,      # the row mover (the sort kernels move < 1 % of that)
-    "moe_unpermute": 3.07,
+    "bf16_m_grouped_gateup_nt": (11.98, "gemm16"),
+    "bf16_m_grouped_gateup_nn": (11.94, "gemm16"),
+    "bf16_m_grouped_gateup_fp8_out": (10.69, "gemm16"),
+    "bf16_m_grouped_down_nt": (5.38, "gemm16"),
+    "bf16_m_grouped_down_nn": (5.42, "gemm16"),
+    "bf16_masked_decode": (2.51, "gemm16"),
+    "bf16_k_grouped_wgrad": (28.31, "gemm16"),
+    "fp8_block_m_grouped": (29.07, "gemm8"),
+    "fp8_channel_m_grouped": (27.73, "gemm8"),
+    "fp8_channel_k_grouped": (18.05, "gemm8"),
+    "quant_trans128": (8.12, "quant"),
+    "moe_permute": (3.06, "permute"),      # the row mover (the sort kernels move < 1 % of that)
+    "moe_unpermute": (3.07, "permute"),
 }
+TRAFFIC_SOURCES = {
+    "gemm16": ("common.hpp", "sched.hpp", "fast_common.hpp", "gemm_fast.hip"),
+    "gemm8": ("common.hpp", "sched.hpp", "fast_common.hpp", "gemm_fp8.hip"),
+    "quant": ("common.hpp", "sched.hpp", "quant.hip"),
+    "permute": ("moe_permute.hip",),
+}
+TRAFFIC_STAMPS = {  # sha256 over the source set's files, first 16 hex digits, at the time of the counter runs
+    "gemm16": "",
+    "gemm8": "",
+    "quant": "",
+    "permute": "",
+}
+
+
+def source_stamp(source_set: str) -> str:
+    h = hashlib.sha256()
+    for name in TRAFFIC_SOURCES[source_set]:
+        with open(os.path.join(ROOT, "triton_grouped_gemm_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(name: str):
+    """Bytes per launch from the table above, or None when there is no figure for this workload or the kernel
+    sources have changed since it was measured."""
+    entry = MEASURED_TRAFFIC_GB.get(name)
+    if entry is None:
+        return None
+    gb, source_set = entry
+    try:
+        return round(gb * 1e9) if source_stamp(source_set) == TRAFFIC_STAMPS[source_set] else None
+    except OSError:
+        return None
 
 G, M_TOTAL = 128, 655360
 WORKLOADS = {
@@ -75,6 +122,7 @@ WORKLOADS = {
     "fp8_channel_m_grouped_readme": ("fp8c", 6144, 5120, True, dict(sizes=[509, 3587, 125, 3971] * 8, fmt_a="e5m2")),
     "fp8_channel_k_grouped_readme": ("fp8ck", 6144, 5120, False, dict(sizes=[512, 3584, 128, 3968] * 8, fmt_a="e5m2")),
     "quant_trans128": ("quant", 4096, 0, False),
+    "quant_token128": ("quant1", 0, 4096, False),    # the 1x128 activation quantizer on [M, K] bf16
     # MoE token movement either side of the GEMMs: 81920 tokens x top-8 = 655360 rows of 2048 bf16
     "moe_permute": ("permute", 2048, 8, False),       # hidden, topK
     "moe_unpermute": ("unpermute", 2048, 8, False),
@@ -90,18 +138,23 @@ METRICS = {
     "fp8c": "grouped GEMM TFLOP/s (2*M*N*K/time), FP8 per-channel M-grouped G=128",
     "fp8ck": "grouped GEMM TFLOP/s (2*K_total*M*N/time), FP8 per-channel K-grouped G=128",
     "quant": "transposing 128x128 quantizer, algorithmic GB/s",
+    "quant1": "1x128 activation quantizer (per_token_cast_to_fp8), algorithmic GB/s",
     "permute": "MoE permute (sort + row mover), algorithmic GB/s",
     "unpermute": "MoE unpermute, algorithmic GB/s",
 }
 
 
 def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu: int = -1, uniform: bool = False,
-                   groups: int = None, m_total: int = None):
+                   groups: int = None, m_total: int = None, dtype: str = "bf16", size_mode: str = None,
+                   group_align: int = 64):
     """Returns (fn, flops_per_step, algorithmic_bytes_per_step, dtype_tag, description, cpu_sample_fn); leaves a
     per-group library-GEMM loop over the same operands in ``build_workload.vendor_loop`` where one exists, the
     tensor that loop writes in ``build_workload.vendor_out`` and the operands in ``build_workload.operands``.
     ``uniform``: every group gets m_total / groups rows (the reference's published tables use 128 groups of 5120
-    rows) instead of the Dirichlet-multinomial draw.  ``groups`` / ``m_total`` shrink the problem (tests)."""
+    rows) instead of the Dirichlet-multinomial draw.  ``size_mode`` "random" / "random-unaligned": the draws of the
+    reference's benchmark main for --random-groups (blocks of ``group_align`` rows) / --unaligned-random-groups.
+    ``dtype`` "fp16": 16-bit GEMM workloads on half precision operands.  ``groups`` / ``m_total`` shrink the
+    problem (tests)."""
     build_workload.vendor_loop = None
     build_workload.vendor_out = None
     build_workload.vendor_kind = None
@@ -116,15 +169,25 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
         sizes_cpu = torch.tensor(opts["sizes"], dtype=torch.int32)
         G, M_TOTAL = len(opts["sizes"]), int(sum(opts["sizes"]))
         size_tag = "as the reference's example: " + " ".join(map(str, opts["sizes"][:4])) + f" x {G // 4}"
+    elif size_mode in ("random", "random-unaligned"):
+        sizes_cpu = wl.reference_group_sizes(G, M_TOTAL, seed, False, group_align, size_mode == "random")
+        size_tag = (f"random as the reference's --random-groups, blocks of {group_align} rows" if size_mode == "random"
+                    else "random as the reference's --unaligned-random-groups (exact sum, no alignment)")
     else:
         sizes_cpu = wl.uniform_sizes(G, M_TOTAL) if uniform else wl.dirichlet_multinomial_sizes(G, M_TOTAL, 128, seed=seed)
         size_tag = f"uniform, {M_TOTAL // G} rows per group" if uniform else "dirichlet-multinomial, 128-aligned"
     sizes = sizes_cpu.to(dev)
+    t16 = torch.float16 if dtype == "fp16" else torch.bfloat16
+    tag16 = "fp16" if dtype == "fp16" else "bf16"
+
+    def randn16(shape, scale, sd):  # N(0,1)*scale in the 16-bit type of the run (fp16: the bf16 draw, converted)
+        x = wl.randn_bf16(shape, scale, sd, dev)
+        return x if t16 == torch.bfloat16 else x.to(t16)
     fp8_a = torch.float8_e5m2 if opts.get("fmt_a") == "e5m2" else torch.float8_e4m3fn
     bounds = [(int(s0), int(s0 + n)) for s0, n in zip((sizes_cpu.cumsum(0) - sizes_cpu).tolist(), sizes_cpu.tolist())]
     if kind == "mg":
-        a = wl.randn_bf16((M_TOTAL, K), K ** -0.5, seed + 1, dev)
-        b = wl.randn_bf16((G, N, K) if trans_b else (G, K, N), K ** -0.5, seed + 2, dev)
+        a = randn16((M_TOTAL, K), K ** -0.5, seed + 1)
+        b = randn16((G, N, K) if trans_b else (G, K, N), K ** -0.5, seed + 2)
         if zeros:  # same kernel, same traffic, no switching activity in the multipliers
             a.zero_()
             b.zero_()
@@ -154,8 +217,8 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
                 groups += 1
                 if t_used >= budget_s:
                     break
-            return done_flops / t_used / 1e12, f"{groups} largest groups of {G} ({done_flops / flops * 100:.1f}% of the step's flops), bf16 torch matmul per group"
-        c_ref = torch.empty((M_TOTAL, N), device=dev, dtype=torch.bfloat16)
+            return done_flops / t_used / 1e12, f"{groups} largest groups of {G} ({done_flops / flops * 100:.1f}% of the step's flops), {tag16} torch matmul per group"
+        c_ref = torch.empty((M_TOTAL, N), device=dev, dtype=t16)
 
         def vendor_loop():  # one library GEMM per expert, the GPU baseline the reference's tables compare against
             for g, (s0, s1) in enumerate(bounds):
@@ -163,8 +226,8 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
                     torch.matmul(a[s0:s1], b[g].t() if trans_b else b[g], out=c_ref[s0:s1])
         build_workload.vendor_loop = vendor_loop
         build_workload.vendor_out = c_ref
-        return fn, flops, nbytes, "bf16", dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, trans_b=trans_b,
-                                               group_sizes=size_tag, seed=seed), cpu_sample
+        return fn, flops, nbytes, tag16, dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, trans_b=trans_b,
+                                              group_sizes=size_tag, seed=seed), cpu_sample
     if kind == "mgq":
         from triton_grouped_gemm_amd.gemm.fused import m_grouped_gemm_fp8_out
         a = wl.randn_bf16((M_TOTAL, K), K ** -0.5, seed + 1, dev)
@@ -179,20 +242,20 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
         m_max = 512
         mm_cpu = wl.masked_counts(G, m_max, seed)
         mm = mm_cpu.to(dev)
-        lhs = wl.randn_bf16((G * m_max, K), K ** -0.5, seed + 1, dev)
-        rhs = wl.randn_bf16((G, N, K), K ** -0.5, seed + 2, dev)
-        out = torch.empty((G * m_max, N), device=dev, dtype=torch.bfloat16)
+        lhs = randn16((G * m_max, K), K ** -0.5, seed + 1)
+        rhs = randn16((G, N, K), K ** -0.5, seed + 2)
+        out = torch.empty((G * m_max, N), device=dev, dtype=t16)
         mv = float(mm_cpu.sum())
         fn = lambda: m_grouped_gemm_masked(lhs, rhs, out, mm, m_max)
-        return (fn, 2.0 * mv * N * K, 2.0 * mv * K + 2.0 * int((mm_cpu > 0).sum()) * N * K + 2.0 * mv * N, "bf16",
+        return (fn, 2.0 * mv * N * K, 2.0 * mv * K + 2.0 * int((mm_cpu > 0).sum()) * N * K + 2.0 * mv * N, tag16,
                 dict(workload=name, G=G, m_max=m_max, N=N, K=K, valid_rows=int(mv), seed=seed), None)
     if kind == "kg":
         from triton_grouped_gemm_amd.gemm.BF16.k_grouped_gemm_TMA import k_grouped_gemm
         Nd, Md = N, K
-        a = wl.randn_bf16((M_TOTAL, Md), 1.0, seed + 1, dev)
-        b = wl.randn_bf16((M_TOTAL, Nd), 1.0, seed + 2, dev)
+        a = randn16((M_TOTAL, Md), 1.0, seed + 1)
+        b = randn16((M_TOTAL, Nd), 1.0, seed + 2)
         fn = lambda: k_grouped_gemm(a, b, sizes)
-        c_ref = torch.zeros((G, Md, Nd), device=dev, dtype=torch.bfloat16)
+        c_ref = torch.zeros((G, Md, Nd), device=dev, dtype=t16)
 
         def vendor_loop():
             for g, (s0, s1) in enumerate(bounds):
@@ -200,7 +263,7 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
                     torch.matmul(a[s0:s1].t(), b[s0:s1], out=c_ref[g])
         build_workload.vendor_loop = vendor_loop
         build_workload.vendor_out = c_ref
-        return (fn, 2.0 * M_TOTAL * Md * Nd, 2.0 * M_TOTAL * (Md + Nd) + 2.0 * G * Md * Nd, "bf16",
+        return (fn, 2.0 * M_TOTAL * Md * Nd, 2.0 * M_TOTAL * (Md + Nd) + 2.0 * G * Md * Nd, tag16,
                 dict(workload=name, G=G, K_total=M_TOTAL, M_dim=Md, N_dim=Nd, group_sizes=size_tag, seed=seed), None)
     if kind == "fp8":
         from triton_grouped_gemm_amd.gemm.deep_gemm_ops import m_grouped_fp8_nt_contiguous
@@ -225,9 +288,34 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
         build_workload.vendor_loop = vendor_loop
         build_workload.vendor_out = c_ref
         build_workload.vendor_kind = "torch._scaled_mm per group (hipBLASLt), same fp8 codes, unit scales: no block scaling"
-        return (fn, 2.0 * M_TOTAL * N * K, nbytes, "fp8",
+        flops = 2.0 * M_TOTAL * N * K
+
+        def cpu_sample(budget_s: float):
+            """The oracle's computation for this path on the host cores: dequantise both operands (1x128 and 128x128
+            scales), fp32 matmul, group by group, largest groups first until the time budget is used."""
+            from oracle import gemm_ref
+            order = torch.argsort(sizes_cpu, descending=True).tolist()
+            done_flops, t_used, n_groups = 0.0, 0.0, 0
+            for g in order:
+                s0, s1 = bounds[g]
+                if s1 == s0:
+                    continue
+                ag, sg = aq[0][s0:s1].float().cpu(), aq[1][s0:s1].cpu().contiguous()
+                wg, wsg = wq[0][g:g + 1].float().cpu(), wq[1][g:g + 1].cpu()
+                if n_groups == 0:  # thread pool and allocator warm-up on a few rows
+                    gemm_ref.fp8_block_scaled_reference(ag[:128], sg[:128], wg, wsg, [128])
+                t0 = time.perf_counter()
+                gemm_ref.fp8_block_scaled_reference(ag, sg, wg, wsg, [s1 - s0])
+                t_used += time.perf_counter() - t0
+                done_flops += 2.0 * (s1 - s0) * N * K
+                n_groups += 1
+                if t_used >= budget_s:
+                    break
+            return done_flops / t_used / 1e12, (f"{n_groups} largest groups of {G} ({done_flops / flops * 100:.1f}% of the step's flops), "
+                                                "dequantise + fp32 torch matmul per group")
+        return (fn, flops, nbytes, "fp8",
                 dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, recipe="1x128 act / 128x128 weight, e4m3fn",
-                     group_sizes=size_tag, seed=seed), None)
+                     group_sizes=size_tag, seed=seed), cpu_sample)
     if kind == "fp8c":
         from triton_grouped_gemm_amd.gemm.FP8.m_grouped_gemm_channel_expert import gmm_fp8_act_per_channel_w_per_expert
         gen = torch.Generator(device=dev).manual_seed(seed + 3)
@@ -274,6 +362,12 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
         fn = lambda: trans_per_block_quant_expand_128x(x, sizes)
         nbytes = 2.0 * M_TOTAL * N + 1.0 * N * me + 4.0 * (N / 128) * (me / 128)
         return fn, 0.0, nbytes, "bf16->fp8", dict(workload=name, G=G, M=M_TOTAL, N=N, seed=seed), None
+    if kind == "quant1":
+        from triton_grouped_gemm_amd.quant.fp8_cast import per_token_cast_to_fp8
+        x = wl.randn_bf16((M_TOTAL, K), 1.0, seed + 1, dev)
+        fn = lambda: per_token_cast_to_fp8(x, scales_mn_major=True)
+        nbytes = 2.0 * M_TOTAL * K + 1.0 * M_TOTAL * K + 4.0 * M_TOTAL * K / 128
+        return fn, 0.0, nbytes, "bf16->fp8", dict(workload=name, M=M_TOTAL, K=K, scales="[K/128, M]", seed=seed), None
     if kind in ("permute", "unpermute"):
         from triton_grouped_gemm_amd import ops
         H, topk = N, K
@@ -312,11 +406,11 @@ def time_workload(fn, steps: int, warmup: int, dev):
     return wall_ms, [s.elapsed_time(e) for s, e in evs]
 
 
-def summarise(name: str, flops: float, nbytes: float, dtype_tag: str, wall_ms: float, kernel_ms, uniform: bool):
-    """(value, unit, roofline dict) of one timed workload."""
+def summarise(name: str, flops: float, nbytes: float, dtype_tag: str, wall_ms: float, kernel_ms, default_draw: bool):
+    """(value, unit, roofline dict) of one timed workload.  ``default_draw``: the workload ran on the group sizes and
+    data type the traffic counters were read on (the Dirichlet draw, bf16): only then is the measured traffic its."""
     avg_kernel_ms = sum(kernel_ms) / len(kernel_ms)
-    traffic = None if uniform else MEASURED_TRAFFIC_GB.get(name)  # measured on the Dirichlet draw only
-    traffic = None if traffic is None else round(traffic * 1e9)  # bytes per launch
+    traffic = measured_traffic(name) if default_draw else None  # bytes per launch, or None
     if flops > 0:
         value = flops / (wall_ms * 1e-3) / 1e12
         peak = PEAK_TFLOPS["fp8" if dtype_tag == "fp8" else "bf16"]
@@ -325,6 +419,15 @@ def summarise(name: str, flops: float, nbytes: float, dtype_tag: str, wall_ms: f
                         frac=round(achieved / peak, 4), traffic=traffic,
                         min_ms=round(min(kernel_ms), 4), avg_ms=round(avg_kernel_ms, 4),
                         algorithmic_gbytes=round(nbytes / 1e9, 3))
+        if WORKLOADS[name][0] == "masked":
+            # Decode-style masked GEMM: about 200 flop per algorithmic byte, below the ridge (312 for bf16), so the HBM
+            # roof is the one that binds.  It is the roofline of the line; the MFMA figure goes beside it.
+            gbs = nbytes / (avg_kernel_ms * 1e-3) / 1e9
+            hbm = dict(bound="hbm", achieved=round(gbs, 1), peak=PEAK_HBM_GBS, unit="GB/s",
+                       frac=round(gbs / PEAK_HBM_GBS, 4), traffic=traffic,
+                       min_ms=round(min(kernel_ms), 4), avg_ms=round(avg_kernel_ms, 4),
+                       algorithmic_gbytes=round(nbytes / 1e9, 3), mfma=roofline)
+            return value, "TFLOP/s", hbm
         return value, "TFLOP/s", roofline
     value = nbytes / (wall_ms * 1e-3) / 1e9
     achieved = nbytes / (avg_kernel_ms * 1e-3) / 1e9
@@ -355,22 +458,135 @@ def time_vendor_loop(flops: float):
                 kind=kind + ", wall time incl. launches")
 
 
+REFERENCE_CASES = [  # the reference's BENCHMARK_CASES (gemm/BF16/m_grouped_gemm_TMA.py:474-493): model, n, k, total_m, trans_b
+    ("30B", 1536, 2048, 655360, True), ("30B", 1536, 2048, 655360, True),
+    ("30B", 1536, 2048, 655360, False), ("30B", 1536, 2048, 655360, False),
+    ("30B", 2048, 768, 655360, True), ("30B", 2048, 768, 655360, True),
+    ("30B", 2048, 768, 655360, False), ("30B", 2048, 768, 655360, False),
+    ("235B", 3072, 4096, 655360, True), ("235B", 3072, 4096, 655360, True),
+    ("235B", 3072, 4096, 655360, False), ("235B", 3072, 4096, 655360, False),
+    ("235B", 4096, 1536, 655360, True), ("235B", 4096, 1536, 655360, True),
+    ("235B", 4096, 1536, 655360, False), ("235B", 4096, 1536, 655360, False),
+]
+
+
+def event_min_avg(fn, warmup: int, active: int):
+    """The reference's ``benchmark_cuda_event`` (gemm/BF16/m_grouped_gemm_TMA.py:584-599): ``warmup`` untimed calls,
+    then ``active`` calls each between two events; (min ms, mean ms)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(active):
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        fn()
+        e.record()
+        e.synchronize()
+        times.append(s.elapsed_time(e))
+    return min(times), sum(times) / len(times)
+
+
+def run_reference_cases(args, dev) -> int:
+    """The reference's benchmark main, case by case, on this library: same cases, flags, group-size draws, operands
+    (unscaled torch.randn), timing and correctness gate (row-max normalisation, assert_close at 1e-2 against the
+    per-group torch matmul); the per-group library GEMM loop stands where its cuBLAS extension stood."""
+    from oracle import gemm_ref
+    from triton_grouped_gemm_amd import workloads as wl
+    from triton_grouped_gemm_amd.gemm.BF16.m_grouped_gemm_TMA import _build_m_grouped_metadata, _m_grouped_gemm_launch
+    torch.manual_seed(args.seed)
+    torch.cuda.manual_seed_all(args.seed)
+    dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float16
+    cases = [c for c in REFERENCE_CASES if args.only_model is None or c[0] == args.only_model]
+    results = []
+    for case_idx, (model, n, k, total_m, trans_b) in enumerate(cases):
+        torch.cuda.empty_cache()
+        sizes_cpu = wl.reference_group_sizes(args.groups, total_m, args.seed + case_idx, not args.random_groups,
+                                             args.group_align, not args.unaligned_random_groups)
+        sizes = sizes_cpu.to(device=dev, dtype=torch.int64)
+        M = int(sizes_cpu.sum())
+        assert M == total_m, f"generated M={M}, expected {total_m}"
+        starts = sizes_cpu.to(torch.int64).cumsum(0) - sizes_cpu
+        bad_8, bad_64 = int((starts % 8 != 0).sum()), int((starts % 64 != 0).sum())
+        metadata = _build_m_grouped_metadata(sizes)
+        a = torch.randn(M, k, dtype=dtype, device=dev)
+        b = torch.randn((args.groups, n, k) if trans_b else (args.groups, k, n), dtype=dtype, device=dev)
+        layout = "B[G,N,K]" if trans_b else "B[G,K,N]"
+        out = torch.empty(M, n, dtype=dtype, device=dev)
+        lib_min, lib_avg = event_min_avg(lambda: _m_grouped_gemm_launch(a, b, out, sizes, trans_b, args.num_sm, metadata=metadata),
+                                         args.warmup, args.active)
+        bounds = [(int(s0), int(s0 + c)) for s0, c in zip(starts.tolist(), sizes_cpu.tolist())]
+        v_min = v_avg = 0.0
+        if not args.skip_vendor:
+            c_ref = torch.empty_like(out)
+
+            def vendor():
+                for g, (s0, s1) in enumerate(bounds):
+                    if s1 > s0:
+                        torch.matmul(a[s0:s1], b[g].t() if trans_b else b[g], out=c_ref[s0:s1])
+            v_min, v_avg = event_min_avg(vendor, args.warmup, args.active)
+            del c_ref
+        if not args.skip_check:  # the reference's gate: m_grouped_reference on the same device, row-max normalised, 1e-2
+            ref = torch.cat([a[s0:s1] @ (b[g].t() if trans_b else b[g]) for g, (s0, s1) in enumerate(bounds) if s1 > s0])
+            torch.testing.assert_close(gemm_ref.row_max_normalization(out.float()), gemm_ref.row_max_normalization(ref.float()),
+                                       rtol=1e-2, atol=1e-2)
+            del ref
+        flops = 2.0 * M * n * k
+        print(f"[{case_idx:02d}] model={model}, n={n}, k={k}, M={M}, trans_b={trans_b}, layout={layout}, out_layout=C[M,N], "
+              f"bad_start_align8={bad_8}/{args.groups}, bad_start_align64={bad_64}/{args.groups}", flush=True)
+        print(f"    HIP kernel GPU time {lib_min:.2f} ms min / {lib_avg:.2f} ms avg, {flops / lib_min / 1e9:.0f} TFLOP/s min-time / "
+              f"{flops / lib_avg / 1e9:.0f} TFLOP/s avg-time", flush=True)
+        if v_min > 0:
+            print(f"    hipBLASLt per-group loop GPU time {v_min:.2f} ms min / {v_avg:.2f} ms avg, {flops / v_min / 1e9:.0f} TFLOP/s; "
+                  f"speedup {v_min / lib_min:.2f}x (baseline_layout={layout})", flush=True)
+        results.append({
+            "case_idx": case_idx, "model": model, "n": n, "k": k, "M": M, "trans_b": trans_b, "layout": layout,
+            "output_layout": "C[M,N]", "groups": args.groups, "dtype": args.dtype,
+            "kernel_min_ms": lib_min, "kernel_avg_ms": lib_avg,
+            "kernel_tflops_min_time": flops / lib_min / 1e9, "kernel_tflops_avg_time": flops / lib_avg / 1e9,
+            "vendor_loop_min_ms": v_min, "vendor_loop_avg_ms": v_avg,
+            "vendor_loop_tflops_min_time": flops / v_min / 1e9 if v_min > 0 else 0.0,
+            "speedup_vs_vendor_loop": v_min / lib_min if v_min > 0 else 0.0,
+            "group_sizes": "uniform" if not args.random_groups else ("random-unaligned" if args.unaligned_random_groups else f"random-align{args.group_align}"),
+            "bad_start_align8": bad_8, "bad_start_align64": bad_64,
+        })
+        del a, b, out
+    if args.csv:
+        os.makedirs(os.path.dirname(os.path.abspath(args.csv)), exist_ok=True)
+        with open(args.csv, "w", newline="") as f:
+            writer = csv.DictWriter(f, fieldnames=list(results[0].keys()))
+            writer.writeheader()
+            writer.writerows(results)
+        print(f"Wrote CSV summary to {args.csv}", flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=12,
-                    help="untimed launches first: the first ten or so run at a clock that is still settling (4.2 -> 3.3 ms on the headline)")
+    ap.add_argument("--warmup", type=int, default=None,
+                    help="untimed launches first (default 12: the first ten or so run at a clock that is still settling, "
+                         "4.2 -> 3.3 ms on the headline; --reference-cases: 5, as the reference)")
     ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS),
-                    help="default: bf16_m_grouped_gateup_nt, followed by fp8_block_m_grouped under the line's \"fp8\" key")
-    ap.add_argument("--uniform-groups", action="store_true",
-                    help="every group gets M / G = 5120 rows, as in the reference's published tables, instead of the "
-                         "Dirichlet-multinomial draw")
-    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="host-core time budget of the CPU baseline sample")
+                    help="default: bf16_m_grouped_gateup_nt, followed by the other configurations of the path under their own keys")
+    ap.add_argument("--dtype", choices=["bf16", "fp16"], default="bf16", help="16-bit GEMM workloads: operand and output type")
+    group_mode = ap.add_mutually_exclusive_group()
+    group_mode.add_argument("--uniform-groups", action="store_true",
+                            help="every group gets M / G = 5120 rows, as in the reference's published tables, instead of the "
+                                 "Dirichlet-multinomial draw (the default of --reference-cases, as in the reference)")
+    group_mode.add_argument("--random-groups", action="store_true",
+                            help="group sizes as the reference's --random-groups draws them, in blocks of --group-align rows")
+    ap.add_argument("--unaligned-random-groups", action="store_true",
+                    help="with --random-groups: exact-sum random sizes without alignment")
+    ap.add_argument("--group-align", type=int, default=64, help="alignment, in rows, of --random-groups sizes")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="host-core time budget of each CPU baseline sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-vendor-loop", action="store_true",
                     help="skip timing the per-group library GEMM loop (hipBLASLt through torch) over the same operands")
     ap.add_argument("--no-fp8", action="store_true", help="default run: skip the FP8 block-scaled half")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="default run: skip the masked, K-grouped and quantizer configurations that follow the two headline halves")
     ap.add_argument("--zeros", action="store_true",
                     help="M-grouped bf16 workloads only: all-zero operands (diagnostic: shows how far the clock is held down "
                          "by the power the multipliers draw on random data); reported as data=synthetic-zeros")
@@ -378,28 +594,71 @@ def main() -> int:
                     help="M-grouped bf16 workloads only: cap the persistent grid at this many workgroups (diagnostic)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy (reference kernel for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--print-traffic-stamps", action="store_true",
+                    help="print the current hashes of the kernel source sets that the measured-traffic table is stamped with")
+    # the reference's benchmark main (gemm/BF16/m_grouped_gemm_TMA.py:602-635), flag for flag
+    ap.add_argument("--reference-cases", action="store_true", help="run the reference's sixteen M-grouped cases and print its per-case lines")
+    ap.add_argument("--groups", type=int, default=128)
+    ap.add_argument("--active", type=int, default=10, help="--reference-cases: timed launches per case")
+    ap.add_argument("--seed", type=int, default=2026)
+    ap.add_argument("--num-sm", type=int, default=-1, help="--reference-cases: cap on the persistent grid (numSM)")
+    ap.add_argument("--skip-check", action="store_true", help="--reference-cases: skip the correctness gate")
+    ap.add_argument("--skip-vendor", "--skip-cublas", dest="skip_vendor", action="store_true",
+                    help="--reference-cases: skip the per-group library GEMM loop (the reference's --skip-cublas)")
+    ap.add_argument("--csv", type=str, default="", help="--reference-cases: write the summary as CSV")
+    ap.add_argument("--only-model", choices=["30B", "235B"], default=None)
     args = ap.parse_args()
+    if args.print_traffic_stamps:
+        print(json.dumps({k: source_stamp(k) for k in TRAFFIC_SOURCES}))
+        return 0
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: the grouped-GEMM path has no cross-GPU step; run with --gpus 1", file=sys.stderr)
         return 2
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (there is no CPU path)", file=sys.stderr)
         return 2
+    if args.unaligned_random_groups and not args.random_groups:
+        print("--unaligned-random-groups goes with --random-groups", file=sys.stderr)
+        return 2
     from triton_grouped_gemm_amd import _native
     _native.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.reference_cases:
+        args.warmup = 5 if args.warmup is None else args.warmup
+        return run_reference_cases(args, dev)
+    args.warmup = 12 if args.warmup is None else args.warmup
     workload = args.workload or "bf16_m_grouped_gateup_nt"
-    with_fp8 = args.workload is None and not args.no_fp8 and not args.zeros and args.num_cu <= 0
+    default_run = args.workload is None and not args.zeros and args.num_cu <= 0
+    with_fp8 = default_run and not args.no_fp8
+    with_extras = default_run and not args.no_extras
     kind = WORKLOADS[workload][0]
     if (args.zeros or args.num_cu > 0) and kind != "mg":
         print("--zeros / --num-cu apply to the bf16_m_grouped_* workloads only", file=sys.stderr)
         return 2
-    if args.uniform_groups and kind in ("masked", "quant", "permute", "unpermute"):
-        print("--uniform-groups applies to the M-grouped and K-grouped GEMM workloads", file=sys.stderr)
+    if (args.uniform_groups or args.random_groups) and kind in ("masked", "quant", "quant1", "permute", "unpermute"):
+        print("--uniform-groups / --random-groups apply to the M-grouped and K-grouped GEMM workloads", file=sys.stderr)
         return 2
-    fn, flops, nbytes, dtype_tag, config, cpu_sample = build_workload(workload, dev, zeros=args.zeros, num_cu=args.num_cu,
-                                                                      uniform=args.uniform_groups)
+    if args.dtype != "bf16" and kind not in ("mg", "masked", "kg"):
+        print("--dtype fp16 applies to the 16-bit M-grouped, masked and K-grouped GEMM workloads", file=sys.stderr)
+        return 2
+    size_mode = None if not args.random_groups else ("random-unaligned" if args.unaligned_random_groups else "random")
+    default_draw = not (args.uniform_groups or args.random_groups) and args.dtype == "bf16" and args.groups == 128
+    groups = None if args.groups == 128 else args.groups
+
+    def build(name):
+        return build_workload(name, dev, seed=args.seed, zeros=args.zeros and name == workload, num_cu=args.num_cu,
+                              uniform=args.uniform_groups, groups=groups, dtype=args.dtype, size_mode=size_mode,
+                              group_align=args.group_align)
+
+    def cpu_base(sample_fn):
+        if sample_fn is None or args.no_cpu_baseline:
+            return None
+        tf, sample = sample_fn(args.cpu_seconds)
+        return dict(value=round(tf, 4), unit="TFLOP/s", cores=torch.get_num_threads(), kind="port", sample=sample,
+                    host_cpus=os.cpu_count())
+
+    fn, flops, nbytes, dtype_tag, config, cpu_sample = build(workload)
     if args.num_cu > 0:
         config["num_cu"] = args.num_cu
 
@@ -410,14 +669,9 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
     wall_ms, kernel_ms = time_workload(fn, args.steps, args.warmup, dev)
-    value, unit, roofline = summarise(workload, flops, nbytes, dtype_tag, wall_ms, kernel_ms, args.uniform_groups)
+    value, unit, roofline = summarise(workload, flops, nbytes, dtype_tag, wall_ms, kernel_ms, default_draw)
     vendor = None if args.no_vendor_loop else time_vendor_loop(flops)
-
-    cpu_baseline = None
-    if cpu_sample is not None and not args.no_cpu_baseline:
-        tf, sample = cpu_sample(args.cpu_seconds)
-        cpu_baseline = dict(value=round(tf, 4), unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
-                            sample=sample, host_cpus=os.cpu_count())
+    cpu_baseline = cpu_base(cpu_sample)
 
     line = {
         "metric": METRICS[kind].replace("G=128", f"G={config['G']}") if "G" in config else METRICS[kind], "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps,
@@ -426,18 +680,33 @@ def main() -> int:
         "roofline": roofline, "cpu_baseline": cpu_baseline, "vendor_loop": vendor,
     }
 
-    if with_fp8:  # the FP8 half of the headline metric: same run, same steps and warm-up, its own operands
-        del fn, cpu_sample
+    def release():
         build_workload.vendor_loop = build_workload.vendor_out = None
         build_workload.operands = {}
         torch.cuda.empty_cache()
+
+    if with_fp8:  # the FP8 half of the headline metric: same run, same steps and warm-up, its own operands
+        del fn, cpu_sample
+        release()
         name8 = "fp8_block_m_grouped"
-        fn8, flops8, nbytes8, tag8, config8, _ = build_workload(name8, dev, uniform=args.uniform_groups)
+        fn8, flops8, nbytes8, tag8, config8, cpu8 = build(name8)
         wall8, kms8 = time_workload(fn8, args.steps, args.warmup, dev)
-        value8, unit8, roof8 = summarise(name8, flops8, nbytes8, tag8, wall8, kms8, args.uniform_groups)
+        value8, unit8, roof8 = summarise(name8, flops8, nbytes8, tag8, wall8, kms8, default_draw)
         line["fp8"] = {"metric": METRICS["fp8"], "value": round(value8, 2), "unit": unit8, "ms_per_step": round(wall8, 4),
                        "dtype": tag8, "config": config8, "roofline": roof8,
-                       "vendor_loop": None if args.no_vendor_loop else time_vendor_loop(flops8)}
+                       "vendor_loop": None if args.no_vendor_loop else time_vendor_loop(flops8),
+                       "cpu_baseline": cpu_base(cpu8)}
+        del fn8, cpu8
+    if with_extras:  # the other configurations of the path, each with its roofline
+        for key, name in (("masked", "bf16_masked_decode"), ("k_grouped", "bf16_k_grouped_wgrad"),
+                          ("quant_trans128", "quant_trans128"), ("quant_token128", "quant_token128")):
+            release()
+            fnx, flopsx, nbytesx, tagx, configx, _ = build(name)
+            wallx, kmsx = time_workload(fnx, args.steps, args.warmup, dev)
+            valuex, unitx, roofx = summarise(name, flopsx, nbytesx, tagx, wallx, kmsx, default_draw)
+            line[key] = {"metric": METRICS[WORKLOADS[name][0]], "value": round(valuex, 2), "unit": unitx,
+                         "ms_per_step": round(wallx, 4), "dtype": tagx, "config": configx, "roofline": roofx}
+            del fnx
     print(json.dumps(line))
     return 0
 

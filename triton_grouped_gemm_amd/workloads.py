@@ -44,3 +44,41 @@ def randn_bf16(shape, scale: float, seed: int, device="cpu") -> torch.Tensor:
     else:
         out.copy_((torch.randn(out.shape, device=device, dtype=torch.float32, generator=gen) * scale).to(torch.bfloat16))
     return out
+
+
+def reference_random_sizes(groups: int, total: int, seed: int = 0) -> list:
+    """Group sizes as the reference's own benchmark draws them for ``--random-groups``
+    (``_fallback_generate_random_list``, gemm/BF16/m_grouped_gemm_TMA.py:496-513): integer weights in [1, 10000)
+    from a seeded CPU generator, sizes proportional to them (floor, at least 1), the remainder dealt out (or taken
+    back from sizes above 1) one row at a time in index order.  Exact sum, no empty group."""
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    weights = torch.randint(1, 10000, (groups,), generator=gen, dtype=torch.int64)
+    sizes = torch.clamp(torch.div(weights * total, weights.sum(), rounding_mode="floor"), min=1).tolist()
+    diff, idx = total - sum(sizes), 0
+    while diff != 0:
+        j = idx % groups
+        if diff > 0:
+            sizes[j] += 1
+            diff -= 1
+        elif sizes[j] > 1:
+            sizes[j] -= 1
+            diff += 1
+        idx += 1
+    return sizes
+
+
+def reference_group_sizes(groups: int, total: int, seed: int, uniform: bool, align: int = 64,
+                          aligned: bool = True) -> torch.Tensor:
+    """``make_group_sizes`` of the reference's benchmark main (gemm/BF16/m_grouped_gemm_TMA.py:541-562): uniform
+    (its default), random in blocks of ``align`` rows (``--random-groups``, :527-538), or random with an exact sum
+    and no alignment (``--unaligned-random-groups``).  int32 on the CPU."""
+    if uniform:
+        assert total % groups == 0, "uniform_groups requires total_m divisible by num_groups"
+        sizes = [total // groups] * groups
+    elif aligned:
+        assert align > 0 and total % align == 0, f"total_m={total} must be divisible by align={align}"
+        assert total // align >= groups, "Need at least one aligned block per group"
+        sizes = [b * align for b in reference_random_sizes(groups, total // align, seed)]
+    else:
+        sizes = reference_random_sizes(groups, total, seed)
+    return torch.tensor(sizes, dtype=torch.int32)
