@@ -321,11 +321,13 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
   // copies of the slab after the next one are issued one per multiply from the barrier on: the sooner they are
   // out, the longer they have to land before the next wait (one per two multiplies measured 3 % slower, two per
   // multiply 4 % slower: the address unit's queue is short, see gemm_fast.hip).
-  // Block scaling: every multiply starts from zero and its result is folded into the accumulators, scaled, two
+  // Block scaling: every multiply starts from zero and its result is folded into the accumulators, scaled, three
   // multiplies later.
   // DEEP: per slab the scale, A and then B copies go out, the B copies for a slab one further ahead; the wait lets
   // the CB most recent copies -- those B copies -- stay in flight (loads complete in order).
   constexpr int WAIT_N = DEEP ? CB : 0;
+  constexpr int kFoldLag = C::TN >= 3 ? 3 : 2;  // block scaling: a product is folded in this many multiplies after its own
+  static_assert(kFoldLag >= 1 && kFoldLag <= 3 && kFoldLag <= C::TN, "four product buffers; the carried products share the last row block's scale");
   if (DEEP) feedb_seek(0);
   feed_seek(0);
   {
@@ -422,7 +424,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
       continue;
     }
 
-    // block scaling: the products that are still to be folded in when a slab ends (those of its last two
+    // block scaling: the products that are still to be folded in when a slab ends (those of its last kFoldLag
     // multiplies) are carried into the next slab
     f32x4_t part[4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
     float s_carry = 0.f;
@@ -484,16 +486,16 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
           }
           if (BLOCK && jj == 0) srow[i] *= sb_cur;
           if (BLOCK) {
-            // fold in the product of the multiply before the previous one (it has had two issue slots to finish;
-            // for n = 0, 1 that is one of the previous slab's last two, scaled with that slab's last row scale).
-            // Four product buffers, indexed by n % 4.  The empty asm statements pin the order (plain arithmetic is
+            // fold in the product of the multiply three back (kFoldLag; for n < 3 that is one of the previous slab's
+            // last three, all of its last row block, scaled with that slab's last row scale).  A lag of two measured
+            // 0.5 % slower, a lag of one 1.7 %; four product buffers, indexed by n % 4, allow up to three.  The empty asm statements pin the order (plain arithmetic is
             // otherwise free to drift, which keeps many products alive at once and spills).
             constexpr int NB = C::TM * C::TN;
             static_assert(NB % 4 == 0, "product buffers are numbered per slab");
-            const int pn = (n + NB - 2) % NB;
+            const int pn = (n + NB - kFoldLag) % NB;
             const int pi = pn / C::TN, pjj = pn % C::TN;
             const int pj = ((pi & 1) && pi != C::TM - 1) ? C::TN - 1 - pjj : pjj;
-            const float sc_prev = n < 2 ? s_carry : srow[pi];
+            const float sc_prev = n < kFoldLag ? s_carry : srow[pi];
             const int pb = pn & 3;
             asm volatile("" : "+v"(part[pb]));
 #pragma unroll
@@ -509,7 +511,7 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
     }
     if (BLOCK) {
 #pragma unroll
-      for (int q = 1; q >= 0; --q) {
+      for (int q = kFoldLag - 1; q >= 0; --q) {
         constexpr int NB = C::TM * C::TN;
         const int pn = NB - 1 - q;
         const int pj = pn % C::TN;  // the last row block runs forward
