@@ -111,6 +111,29 @@ def _unpermute_raw(inp, row_id_map, probs, num_tokens, topk):
     return out
 
 
+def _operand(op: str, name: str, t, device, dtype=None, recommended: str = ""):
+    """One tensor argument of a permute / unpermute call brought into the form the kernels take: on the activations'
+    device, of the index / probability type, contiguous.  Each adjustment is announced with the warning the
+    reference's wrappers give for it (grouped_gemm/grouped_gemm/ops.py:60-92, :178-214), so callers see the same
+    diagnostics; nothing is done to a tensor that already conforms."""
+    if t.is_cpu:
+        warnings.warn(f"The input `{name}` of {op} op is on the device: CPU!")
+        t = t.to(device)
+    if dtype is not None and t.dtype != dtype:
+        warnings.warn(f"The data type of the input `{name}` of {op} op is {t.dtype}! The recommended type is {recommended}.")
+        t = t.to(dtype)
+    if not t.is_contiguous():
+        warnings.warn(f"The input `{name}` of {op} op is discontiguous!")
+        t = t.contiguous()
+    return t
+
+
+def _activations(op: str, t):
+    if t.is_cpu:
+        raise RuntimeError(f"[Error] The input `input_act` of {op} op is on the device: CPU!")
+    return _operand(op, "input_act", t, t.device)
+
+
 class PermuteMoE_topK(torch.autograd.Function):
     """grouped_gemm/grouped_gemm/ops.py:52-160.  The workspace the reference keeps between calls is not needed."""
 
@@ -118,26 +141,13 @@ class PermuteMoE_topK(torch.autograd.Function):
     def forward(ctx, input_act, indices, num_out_tokens, max_token_num, num_experts=MAX_EXPERTS):
         if not input_act.numel():
             return input_act, None
-        if indices.dim() == 1:
-            indices = indices.view(-1, 1)
-        if input_act.is_cpu:
-            raise RuntimeError("[Error] The input `input_act` of permute_topK op is on the device: CPU!")
-        if indices.is_cpu:
-            warnings.warn("The input `indices` of permute_topK op is on the device: CPU!")
-            indices = indices.to(input_act.device)
+        op = "permute_topK"
+        input_act = _activations(op, input_act)
+        indices = indices.view(-1, 1) if indices.dim() == 1 else indices
         if input_act.size(0) != indices.size(0):
-            raise RuntimeError(f"[Error] permute_topK op input `indices` shape mismatch! "
+            raise RuntimeError(f"[Error] {op} op input `indices` shape mismatch! "
                                f"Expect {input_act.size(0)}, but got {indices.size(0)}.")
-        if indices.dtype != torch.int32:
-            warnings.warn(f"The data type of the input `indices` of permute_topK op is {indices.dtype}! "
-                          "The recommended type is torch.int32.")
-            indices = indices.to(torch.int32)
-        if not input_act.is_contiguous():
-            warnings.warn("The input `input_act` of permute_topK op is discontiguous!")
-            input_act = input_act.contiguous()
-        if not indices.is_contiguous():
-            warnings.warn("The input `indices` of permute_topK op is discontiguous!")
-            indices = indices.contiguous()
+        indices = _operand(op, "indices", indices, input_act.device, torch.int32, "torch.int32")
         tokens, topk = indices.shape
         row_id_map, _ = permute_map(indices, num_out_tokens, num_experts)
         n_out = num_out_tokens if num_out_tokens > 0 else tokens * topk
@@ -166,36 +176,15 @@ class UnpermuteMoE_topK(torch.autograd.Function):
         if not input_act.numel():
             ctx.probs = probs
             return input_act
-        if input_act.is_cpu:
-            raise RuntimeError("[Error] The input `input_act` of unpermute_topK op is on the device: CPU!")
-        if row_id_map.is_cpu:
-            warnings.warn("The input `row_id_map` of unpermute_topK op is on the device: CPU!")
-            row_id_map = row_id_map.to(input_act.device)
-        if probs is not None and probs.is_cpu:
-            warnings.warn("The input `probs` of unpermute_topK op is on the device: CPU!")
-            probs = probs.to(input_act.device)
-        if probs is not None and row_id_map.size(0) != probs.size(0) * probs.size(1):
-            raise RuntimeError(f"[Error] unpermute_topK op input `probs` shape mismatch! "
+        op = "unpermute_topK"
+        input_act = _activations(op, input_act)
+        if probs is not None and row_id_map.size(0) != probs.numel():
+            raise RuntimeError(f"[Error] {op} op input `probs` shape mismatch! "
                                f"Expect {row_id_map.size(0)}, but got {probs.size(0) * probs.size(1)}.")
-        if row_id_map.dtype != torch.int32:
-            warnings.warn(f"The data type of the input `row_id_map` of unpermute_topK op is {row_id_map.dtype}! "
-                          "The recommended type is torch.int32.")
-            row_id_map = row_id_map.to(torch.int32)
-        if probs is not None and probs.dtype != torch.float32:
-            warnings.warn(f"The data type of the input `probs` of unpermute_topK op is {probs.dtype}! "
-                          "The recommended type is torch.float32.")
-            probs = probs.to(torch.float32)
-        if not input_act.is_contiguous():
-            warnings.warn("The input `input_act` of unpermute_topK op is discontiguous!")
-            input_act = input_act.contiguous()
-        if not row_id_map.is_contiguous():
-            warnings.warn("The input `row_id_map` of unpermute_topK op is discontiguous!")
-            row_id_map = row_id_map.contiguous()
-        if probs is not None and not probs.is_contiguous():
-            warnings.warn("The input `probs` of unpermute_topK op is discontiguous!")
-            probs = probs.contiguous()
-        num_tokens = probs.size(0) if probs is not None else input_act.size(0)
-        topk = probs.size(1) if probs is not None else 1
+        row_id_map = _operand(op, "row_id_map", row_id_map, input_act.device, torch.int32, "torch.int32")
+        if probs is not None:
+            probs = _operand(op, "probs", probs, input_act.device, torch.float32, "torch.float32")
+        num_tokens, topk = (probs.size(0), probs.size(1)) if probs is not None else (input_act.size(0), 1)
         out = _unpermute_raw(input_act, row_id_map, probs, num_tokens, topk)
         ctx.save_for_backward(input_act, row_id_map, probs)
         ctx.topk = topk
