@@ -46,17 +46,18 @@ PEAK_HBM_GBS = 8000.0
 # printed only while the hash of that source set still equals the stamp below; after any change to those files it
 # is null until the counters are read again (python bench.py --print-traffic-stamps prints the current hashes).
 MEASURED_TRAFFIC_GB = {
-    "bf16_m_grouped_gateup_nt": (11.98, "gemm16"),
-    "bf16_m_grouped_gateup_nn": (11.94, "gemm16"),
-    "bf16_m_grouped_gateup_fp8_out": (10.69, "gemm16"),
-    "bf16_m_grouped_down_nt": (5.38, "gemm16"),
-    "bf16_m_grouped_down_nn": (5.42, "gemm16"),
-    "bf16_masked_decode": (2.51, "gemm16"),
-    "bf16_k_grouped_wgrad": (28.31, "gemm16"),
-    "fp8_block_m_grouped": (29.07, "gemm8"),
-    "fp8_channel_m_grouped": (27.73, "gemm8"),
-    "fp8_channel_k_grouped": (18.05, "gemm8"),
+    "bf16_m_grouped_gateup_nt": (11.85, "gemm16"),
+    "bf16_m_grouped_gateup_nn": (11.79, "gemm16"),
+    "bf16_m_grouped_gateup_fp8_out": (10.82, "gemm16"),
+    "bf16_m_grouped_down_nt": (5.39, "gemm16"),
+    "bf16_m_grouped_down_nn": (5.38, "gemm16"),
+    "bf16_masked_decode": (2.49, "gemm16"),
+    "bf16_k_grouped_wgrad": (28.06, "gemm16"),
+    "fp8_block_m_grouped": (25.84, "gemm8"),
+    "fp8_channel_m_grouped": (28.34, "gemm8"),
+    "fp8_channel_k_grouped": (17.16, "gemm8"),
     "quant_trans128": (8.12, "quant"),
+    "quant_token128": (8.2, "quant"),
     "moe_permute": (3.06, "permute"),      # the row mover (the sort kernels move < 1 % of that)
     "moe_unpermute": (3.07, "permute"),
 }
@@ -67,10 +68,10 @@ TRAFFIC_SOURCES = {
     "permute": ("moe_permute.hip",),
 }
 TRAFFIC_STAMPS = {  # sha256 over the source set's files, first 16 hex digits, at the time of the counter runs
-    "gemm16": "",
-    "gemm8": "",
-    "quant": "",
-    "permute": "",
+    "gemm16": "6e0f56acecfa6b5d",
+    "gemm8": "1de6dfbfb67b2cf3",
+    "quant": "cafd5b44bb56a67c",
+    "permute": "0231abd86ff30831",
 }
 
 
@@ -121,6 +122,9 @@ WORKLOADS = {
     # weights e4m3fn; the K-grouped one with every expert's tokens padded to a multiple of 128.
     "fp8_channel_m_grouped_readme": ("fp8c", 6144, 5120, True, dict(sizes=[509, 3587, 125, 3971] * 8, fmt_a="e5m2")),
     "fp8_channel_k_grouped_readme": ("fp8ck", 6144, 5120, False, dict(sizes=[512, 3584, 128, 3968] * 8, fmt_a="e5m2")),
+    # the headline's shape as ONE dense GEMM through the vendor library (torch.matmul -> hipBLASLt): the whole A against
+    # one expert's weights.  Not a grouped GEMM: the yardstick for what this silicon gives a dense kernel on this shape.
+    "vendor_dense_gateup": ("dense", 1536, 2048, True),
     "quant_trans128": ("quant", 4096, 0, False),
     "quant_token128": ("quant1", 0, 4096, False),    # the 1x128 activation quantizer on [M, K] bf16
     # MoE token movement either side of the GEMMs: 81920 tokens x top-8 = 655360 rows of 2048 bf16
@@ -137,6 +141,7 @@ METRICS = {
     "fp8": "grouped GEMM TFLOP/s (2*M*N*K/time), FP8 block-scaled M-grouped G=128",
     "fp8c": "grouped GEMM TFLOP/s (2*M*N*K/time), FP8 per-channel M-grouped G=128",
     "fp8ck": "grouped GEMM TFLOP/s (2*K_total*M*N/time), FP8 per-channel K-grouped G=128",
+    "dense": "vendor library dense GEMM TFLOP/s (2*M*N*K/time), torch.matmul on the headline's shape",
     "quant": "transposing 128x128 quantizer, algorithmic GB/s",
     "quant1": "1x128 activation quantizer (per_token_cast_to_fp8), algorithmic GB/s",
     "permute": "MoE permute (sort + row mover), algorithmic GB/s",
@@ -156,6 +161,7 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
     ``dtype`` "fp16": 16-bit GEMM workloads on half precision operands.  ``groups`` / ``m_total`` shrink the
     problem (tests)."""
     build_workload.vendor_loop = None
+    build_workload.vendor_dense = None
     build_workload.vendor_out = None
     build_workload.vendor_kind = None
     build_workload.operands = {}
@@ -226,8 +232,20 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
                     torch.matmul(a[s0:s1], b[g].t() if trans_b else b[g], out=c_ref[s0:s1])
         build_workload.vendor_loop = vendor_loop
         build_workload.vendor_out = c_ref
+        # the same shape as one dense GEMM: the whole A against the first expert's weights
+        build_workload.vendor_dense = lambda: torch.matmul(a, b[0].t() if trans_b else b[0], out=c_ref)
         return fn, flops, nbytes, tag16, dict(workload=name, G=G, M=M_TOTAL, N=N, K=K, trans_b=trans_b,
                                               group_sizes=size_tag, seed=seed), cpu_sample
+    if kind == "dense":
+        a = randn16((M_TOTAL, K), K ** -0.5, seed + 1)
+        w = randn16((N, K), K ** -0.5, seed + 2)
+        if zeros:
+            a.zero_()
+            w.zero_()
+        c = torch.empty((M_TOTAL, N), device=dev, dtype=t16)
+        fn = lambda: torch.matmul(a, w.t(), out=c)
+        return (fn, 2.0 * M_TOTAL * N * K, 2.0 * M_TOTAL * K + 2.0 * N * K + 2.0 * M_TOTAL * N, tag16,
+                dict(workload=name, M=M_TOTAL, N=N, K=K, kernel="torch.matmul (hipBLASLt), one dense GEMM", seed=seed), None)
     if kind == "mgq":
         from triton_grouped_gemm_amd.gemm.fused import m_grouped_gemm_fp8_out
         a = wl.randn_bf16((M_TOTAL, K), K ** -0.5, seed + 1, dev)
@@ -437,6 +455,18 @@ def summarise(name: str, flops: float, nbytes: float, dtype_tag: str, wall_ms: f
     return value, "GB/s", roofline
 
 
+def time_vendor_dense(flops: float, steps: int, warmup: int, dev):
+    """The workload's shape as one dense vendor-library GEMM (left behind by build_workload for the M-grouped 16-bit
+    workloads), event-timed like the library's own launches; None where there is none."""
+    vd = getattr(build_workload, "vendor_dense", None)
+    if vd is None:
+        return None
+    _, kms = time_workload(vd, steps, warmup, dev)
+    avg = sum(kms) / len(kms)
+    return dict(value=round(flops / (avg * 1e-3) / 1e12, 2), unit="TFLOP/s", avg_ms=round(avg, 4), min_ms=round(min(kms), 4),
+                kind="torch.matmul (hipBLASLt): the whole A against one expert's weights, i.e. the same M x N x K as ONE dense GEMM")
+
+
 def time_vendor_loop(flops: float):
     """The per-group library-GEMM loop that build_workload left behind, or None (also when the library refuses the call)."""
     vl = build_workload.vendor_loop
@@ -633,13 +663,13 @@ def main() -> int:
     with_fp8 = default_run and not args.no_fp8
     with_extras = default_run and not args.no_extras
     kind = WORKLOADS[workload][0]
-    if (args.zeros or args.num_cu > 0) and kind != "mg":
-        print("--zeros / --num-cu apply to the bf16_m_grouped_* workloads only", file=sys.stderr)
+    if (args.zeros and kind not in ("mg", "dense")) or (args.num_cu > 0 and kind != "mg"):
+        print("--zeros applies to the bf16_m_grouped_* and vendor_dense_* workloads, --num-cu to bf16_m_grouped_* only", file=sys.stderr)
         return 2
     if (args.uniform_groups or args.random_groups) and kind in ("masked", "quant", "quant1", "permute", "unpermute"):
         print("--uniform-groups / --random-groups apply to the M-grouped and K-grouped GEMM workloads", file=sys.stderr)
         return 2
-    if args.dtype != "bf16" and kind not in ("mg", "masked", "kg"):
+    if args.dtype != "bf16" and kind not in ("mg", "masked", "kg", "dense"):
         print("--dtype fp16 applies to the 16-bit M-grouped, masked and K-grouped GEMM workloads", file=sys.stderr)
         return 2
     size_mode = None if not args.random_groups else ("random-unaligned" if args.unaligned_random_groups else "random")
@@ -671,6 +701,7 @@ def main() -> int:
     wall_ms, kernel_ms = time_workload(fn, args.steps, args.warmup, dev)
     value, unit, roofline = summarise(workload, flops, nbytes, dtype_tag, wall_ms, kernel_ms, default_draw)
     vendor = None if args.no_vendor_loop else time_vendor_loop(flops)
+    vendor_dense = None if args.no_vendor_loop else time_vendor_dense(flops, args.steps, args.warmup, dev)
     cpu_baseline = cpu_base(cpu_sample)
 
     line = {
@@ -679,9 +710,11 @@ def main() -> int:
         "vs_baseline": None, "dtype": dtype_tag, "data": "synthetic-zeros" if args.zeros else "synthetic", "config": config,
         "roofline": roofline, "cpu_baseline": cpu_baseline, "vendor_loop": vendor,
     }
+    if vendor_dense is not None:
+        line["vendor_dense"] = vendor_dense
 
     def release():
-        build_workload.vendor_loop = build_workload.vendor_out = None
+        build_workload.vendor_loop = build_workload.vendor_out = build_workload.vendor_dense = None
         build_workload.operands = {}
         torch.cuda.empty_cache()
 
