@@ -68,7 +68,7 @@ def test_tuned_equals_generic_on_random_shapes(dev, seed):
                 try:
                     out4 = m_grouped_gemm(a, b, st, tb)
                 finally:
-                    _native.set_option("four_wave", 0)
+                    _native.set_option("four_wave", 1)
                 assert torch.equal(out4, ref), f"four-wave kernel differs: seed {seed} case {case} G={G} N={N} K={K} {dt}"
             start = 0
             for g, n_rows in enumerate(sizes):  # and against torch's fp32 product, group by group

@@ -113,3 +113,50 @@ def test_built_kernels_have_no_unspaced_hazard():
     for f in files:
         found = scan(f.read_text())
         assert not found, f"{f.name}: {len(found)} hazards, first: {found[0]}"
+
+
+# The four-wave kernel keeps operand chunks that are in flight across loop iterations in v[192:255], named in the
+# text of its own load and LDS-write statements; the compiler must never have allocated one of them for itself (it
+# would move or overwrite a value it knows nothing about).
+_RESERVED = set(range(192, 256))
+
+
+def stray_uses_of_reserved_registers(text: str):
+    """Lines of the four-wave kernels that touch v192..v255 other than the staging loads and LDS writes."""
+    stray, inside = [], False
+    for raw in text.splitlines():
+        line = raw.split(";")[0].strip()
+        if line.endswith(":") and not line.startswith("."):
+            inside = "gemm_w4_kernel" in line
+            continue
+        if not inside or not line or line.startswith("."):
+            continue
+        toks = [t.strip(",") for t in line.split()]
+        used = set().union(*[_regs(t, "v") for t in toks[1:]]) & _RESERVED
+        if not used:
+            continue
+        staged_load = toks[0] == "buffer_load_dwordx4" and _regs(toks[1], "v") == used and toks[-1] != "lds"
+        staged_write = toks[0] == "ds_write_b128" and _regs(toks[2], "v") == used
+        if not (staged_load or staged_write):
+            stray.append(line)
+    return stray
+
+
+def test_reserved_register_scanner_on_snippets():
+    head = "_ZN3tgg14gemm_w4_kernelILi0ELi0EEEvNS_10GemmParamsE:\n"
+    assert stray_uses_of_reserved_registers(head + "buffer_load_dwordx4 v[192:195], v130, s[12:15], s85 offen\n") == []
+    assert stray_uses_of_reserved_registers(head + "ds_write_b128 v146, v[252:255] offset:0x7000\n") == []
+    assert len(stray_uses_of_reserved_registers(head + "v_mov_b32_e32 v200, v3\n")) == 1
+    assert len(stray_uses_of_reserved_registers(head + "v_add_u32_e32 v3, v3, v255\n")) == 1
+    assert len(stray_uses_of_reserved_registers(head + "ds_write_b128 v192, v[4:7]\n")) == 1  # as the address
+    assert stray_uses_of_reserved_registers("other_kernel:\nv_mov_b32_e32 v200, v3\n") == []
+
+
+def test_four_wave_kernel_keeps_its_reserved_registers_to_itself():
+    f = BUILD / "gemm_w4.gfx950.s"
+    if not f.exists():
+        pytest.skip("no device assembly in the build directory (the library was built elsewhere or not yet)")
+    text = f.read_text()
+    assert "gemm_w4_kernel" in text
+    stray = stray_uses_of_reserved_registers(text)
+    assert not stray, f"{len(stray)} compiler-generated uses of v[192:255], first: {stray[0]}"

@@ -22,7 +22,7 @@ static std::atomic<int> g_tile_split{1};
 static std::atomic<int> g_store_nt{1};
 static std::atomic<int> g_n_chunk{0};
 static std::atomic<int> g_kg_second_launch{1};
-static std::atomic<int> g_four_wave{0};  // 0 = eight-wave kernels only, 1 = four-wave kernel on large M-grouped NT launches, 2 = on every launch it can take
+static std::atomic<int> g_four_wave{1};  // 0 = eight-wave kernels only, 1 = four-wave kernel on large M-grouped NT launches (default), 2 = on every launch it can take
 
 int set_error(const char* fmt, ...) {
   va_list ap;

@@ -1,32 +1,43 @@
-// Four-wave bf16/fp16 grouped GEMM kernel for gfx950: the large-problem path of the M-grouped entry points.
+// Four-wave bf16/fp16 grouped GEMM kernel for gfx950: the large-problem path of the M-grouped NT entry points.
 //
 // One workgroup per CU, four waves, one per SIMD; tile 256x256, K slab 64; every wave owns a 128x128 block of
 // 16x16x32 MFMA tiles with its 256 accumulator registers in AGPRs.  Against the eight-wave kernel (gemm_fast.hip,
-// 128x64 per wave) a K step needs a third fewer LDS fragment reads per multiply, and with a single wave per SIMD
-// there is nobody to interleave with, so the instruction order *is* the schedule: the slab loop is written as a
-// sequence of inline-assembly statements (multiplies, fragment reads, direct-to-LDS copies, waits), which the
-// compiler keeps in source order and only allocates registers for.  Measured in isolation on random operands
-// (all 256 CUs, cache-resident source): 1.29 us per 256x256x64 slab against 1.41 us for the eight-wave loop.
+// 128x64 per wave) a K step needs a third fewer LDS fragment reads per multiply.  With a single wave per SIMD there
+// is nobody to interleave with, so the instruction order *is* the schedule: the slab loop is a sequence of
+// inline-assembly statements (multiplies, fragment reads, copies, waits), which the compiler keeps in source order and
+// only allocates registers for.  What the order has to respect (measured with a stream of multiplies and one kind
+// of instruction between them): a wave issues in order and a multiply keeps the matrix pipe busy for 16 cycles, so
+// one or two other instructions between two multiplies cost nothing, three or four cost 4-10 cycles of pipe time,
+// and a 16-byte-per-lane LDS write costs 13 cycles on its own (33 next to fragment reads).  Hence: never more than
+// two instructions in a gap, m0 written a multiply ahead of the copy that needs it, every per-copy address in a
+// register or an immediate, and the per-slab bookkeeping down to an offset and three selects per cursor.
 //
-// Per slab r (two LDS slab buffers, r % 2), per wave:
-//   K step 0   64 multiplies on fragment set 0; meanwhile the 16 fragments of K step 1 are read into set 1
-//   wait for those reads and for this wave's copies of slab r+1, workgroup barrier
+// Per slab r (two LDS slab buffers, r % 2; two register sets for A chunks), per wave:
+//   K step 0   64 multiplies on fragment set 0; meanwhile the 16 fragments of K step 1 are read into set 1, the A
+//              chunks of slab r+1 go from their register set to LDS and the A chunks of slab r+3 are requested
+//              into that set
+//   wait for the fragment reads and for this wave's B copies of slab r+1, workgroup barrier
 //   K step 1   64 multiplies on set 1; meanwhile the fragments of slab r+1 / K step 0 are read into set 0 and
-//              this wave's 16 copies of slab r+2 go out into the buffer of slab r
-// Fragment reads are issued every third multiply, so the last one is a quarter of a K step old when it is
-// waited for; copies every fourth multiply (the address unit takes 16 cycles per copy and its queue is short).
-// The slabs of all of a workgroup's tiles form one stream, as in gemm_fast.hip.
+//              this wave's B copies of slab r+2 go straight to LDS, into the buffer of slab r
+// A is the operand that streams from memory (B panels are shared through L2), so it is requested two slabs
+// earlier than an LDS buffer is free for it: worth 3 % over copying it straight to LDS a slab ahead, although
+// the LDS writes cost more than that copy would.  The slabs of all of a workgroup's tiles form one stream; each
+// of the two cursors carries the buffer descriptor of its tile's window and an offset along K.
 //
 // The epilogue is deferred: a tile's results are converted, staged and stored between the multiplies of the next
 // tile's first K step (see "deferred epilogue" below), whose multiplies start from a zero addend instead of the
-// accumulators.  With one wave per SIMD an epilogue of its own leaves the matrix pipe idle for 12 us per tile
-// (headline 3.88 ms); deferred, conversion and staging disappear under the multiplies (what remains, 0.2 ms per
-// launch, is the issue of the stores themselves): headline 3.43 ms, K = 768 shape 2.78 -> 2.09 ms.  The eight-wave
-// kernel stands at 3.36 / 2.01 ms, so this kernel stays an opt-in path.
+// accumulators.  That K step is the one place where a gap holds a dozen instructions (8 % of a launch).
+//
+// Headline shape (G = 128, M = 655360, N = 1536, K = 2048), same box: 3.18 ms against 3.30 ms for the eight-wave
+// kernel; K = 768 shape 1.91 against 1.97 ms.  Large launches with K a multiple of 128 take this kernel
+// (w4_supported), everything else the eight-wave kernels.
 //
 // What the compiler does not know about assembly statements, and how it is handled here:
 //   * a fragment read's result arrives later: every register a read targets passes through the wait statement
 //     ("+v") before a multiply may use it;
+//   * the A chunks are in flight across loop iterations and paths that join: their registers (v[192:255]) are named
+//     in the instruction text and listed as clobbered, the compiler never holds a value in them
+//     (tests/test_isa_hazards.py scans the kept assembly for any other use);
 //   * the multiplies write AGPRs: compiled code (the epilogue's conversions) reads a block's accumulators no sooner
 //     than 48 multiplies after the multiply that wrote them, except where a flush follows a tile directly: there the
 //     last row block's accumulators pass through a statement of idle cycles first.  Accumulators are never the
@@ -38,7 +49,7 @@ namespace tgg {
 
 namespace {
 
-enum : int { W4_NT = 0, W4_NN = 1 };
+enum : int { W4_NT = 0 };
 constexpr int BK4 = 64;
 
 template <int DT> TGG_DEV void mfma_acc(f32x4_t& acc, const i32x4_t& w, const i32x4_t& x) {
@@ -56,14 +67,6 @@ template <int DT> TGG_DEV void mfma_new(f32x4_t& acc, const i32x4_t& w, const i3
 template <int OFF> TGG_DEV void lds_read_b128(i32x4_t& dst, uint32_t addr) {
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
 }
-// fragment of a token-row operand: two transposing 8-byte reads (K 0..3 and 4..7 of the lane's column)
-template <int OFF0, int OFF1> TGG_DEV void lds_read_tr(i32x4_t& dst, uint32_t addr) {
-  i32x2_t lo, hi;
-  asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
-               : "=&v"(lo), "=&v"(hi) : "v"(addr), "n"(OFF0), "n"(OFF1) : "memory");
-  dst = __builtin_shufflevector(lo, hi, 0, 1, 2, 3);
-}
-
 #define TGG_TIE8(f) "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]), "+v"(f[6]), "+v"(f[7])
 
 struct W4Cfg {
@@ -83,9 +86,8 @@ struct W4Cfg {
 template <int DT, int LAYOUT>
 __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParams p) {
   typedef W4Cfg C;
-  constexpr bool B_KMAJOR = LAYOUT == W4_NT;
-  typedef Operand<C::BM, true> OpA;
-  typedef Operand<C::BN, B_KMAJOR> OpB;
+  static_assert(LAYOUT == W4_NT, "both operands K-contiguous");
+  typedef Operand<C::BM, true> Op;  // A and B slabs have the same geometry: 256 rows of 128 bytes
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::SCHED_OFF);
@@ -98,116 +100,103 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   const int wm0 = (wave >> 1) * 128, wn0 = (wave & 1) * 128;
   const int l16 = lane & 15, lg = lane >> 4;
 
-  const int a_ld = p.K * 2;                                     // global row pitches in bytes
-  const int b_ld = (B_KMAJOR ? p.K : p.N) * 2;
-  // per-lane source offsets of this wave's copies: copy k of an operand is instruction wave + 4 k of the slab, and
-  // the swizzle pattern of an instruction repeats with period NPAT
-  int a_voff[2], b_voff[2], a_voff_tail[2], b_voff_tail[2];
-  const int tail_chunks = (p.K % BK4) / 8;  // K tail: chunks at or beyond K fetch nothing in a tile's last slab
+  const int ld = p.K * 2;  // row pitch of A and of B in bytes; K is a multiple of 128 (w4_supported)
+  // Copy k (0..7) of an operand's slab by this wave is copy instruction wave + 4 k of the slab: rows 8 (wave + 4 k) ...
+  // + 7.  Its per-lane source offset within the tile's window is fixed for the launch; the slab's offset along K
+  // travels in the instruction's scalar offset, which the range check of the window (its valid rows) leaves out.
+  int vo[8];
 #pragma unroll
-  for (int q = 0; q < 2; ++q) {
-    a_voff[q] = OpA::lane_voff(lane, (wave + 4 * q) % OpA::NPAT, a_ld);
-    b_voff[q] = OpB::lane_voff(lane, (wave + 4 * q) % OpB::NPAT, b_ld);
-    a_voff_tail[q] = OpA::lane_chunk(lane, (wave + 4 * q) % OpA::NPAT) >= tail_chunks ? kNoFetch : a_voff[q];
-    b_voff_tail[q] = (B_KMAJOR && OpB::lane_chunk(lane, (wave + 4 * q) % OpB::NPAT) >= tail_chunks) ? kNoFetch : b_voff[q];
-  }
-  static_assert(OpA::NPAT <= 8 && OpB::NPAT <= 8 && 8 % OpA::NPAT == 0 && 8 % OpB::NPAT == 0, "two patterns per wave");
+  for (int k = 0; k < 8; ++k) vo[k] = Op::lane_voff(lane, wave % Op::NPAT, ld) + (wave + 4 * k) * Op::RPI * ld;
+  static_assert(Op::NPAT == 2, "the swizzle pattern of copy wave + 4 k is that of copy wave");
 
-  // LDS addresses of the fragment reads relative to a slab buffer (see gemm_fast.hip for the layouts)
-  uint32_t a_rd[2], b_rd[B_KMAJOR ? 2 : C::TN];
+  // LDS addresses of the fragment reads relative to a slab buffer (see gemm_fast.hip for the layout)
+  uint32_t a_rd[2], b_rd[2];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) a_rd[ks] = smem_addr + (wm0 + l16) * 128 + (((4 * ks + lg) ^ ((l16 / 2) % 8)) << 4);
-  if (B_KMAJOR) {
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
-      b_rd[ks] = smem_addr + C::A_BYTES + (wn0 + l16) * 128 + (((4 * ks + lg) ^ ((l16 / 2) % 8)) << 4);
-  } else {
-#pragma unroll
-    for (int j = 0; j < C::TN; ++j) {
-      const int e = l16 >> 2, c = l16 & 3;
-      const int chunk = ((wn0 + 16 * j) / 8 + (c >> 1)) ^ (e * 4) ^ ((lg & 1) * 2);
-      b_rd[B_KMAJOR ? 0 : j] = smem_addr + C::A_BYTES + (lg * 8 + e) * (C::BN * 2) + chunk * 16 + (c & 1) * 8;
-    }
+  for (int ks = 0; ks < 2; ++ks) {
+    a_rd[ks] = smem_addr + (wm0 + l16) * 128 + (((4 * ks + lg) ^ ((l16 / 2) % 8)) << 4);
+    b_rd[ks] = smem_addr + C::A_BYTES + (wn0 + l16) * 128 + (((4 * ks + lg) ^ ((l16 / 2) % 8)) << 4);
   }
 
-  // ---- the copy stream (as in gemm_fast.hip) ---------------------------------------------------------------------
-  struct TileIo {
-    uint64_t a_base, b_base;
-    int a_rem, b_rem, b_off;
-    int kt_n, issued;
-  };
-  const int kt_all = (p.K + BK4 - 1) / BK4;
-  const int64_t b_step = B_KMAJOR ? BK4 * 2 : (int64_t)BK4 * b_ld;
-  auto make_io = [&](const Tile& t) {
-    TileIo io;
-    io.a_base = uniform64((uint64_t)p.A + (uint64_t)(t.row0 * a_ld));
-    io.a_rem = __builtin_amdgcn_readfirstlane(t.rows * a_ld);  // only the tile's valid rows are fetched
-    io.b_off = 0;
-    if (B_KMAJOR) {
-      const int n_left = p.N - t.n0;
-      io.b_base = uniform64((uint64_t)p.B + (uint64_t)(((int64_t)t.g * p.N + t.n0) * b_ld));
-      io.b_rem = __builtin_amdgcn_readfirstlane((n_left < C::BN ? n_left : C::BN) * b_ld);
-    } else {
-      io.b_base = uniform64((uint64_t)p.B + (uint64_t)((int64_t)t.g * p.K * b_ld + (int64_t)t.n0 * 2));
-      io.b_rem = p.K;
-      io.b_off = __builtin_amdgcn_readfirstlane(t.n0 * 2);
-    }
-    io.kt_n = kt_all;
-    io.issued = 0;
-    return io;
+  // ---- the copy stream --------------------------------------------------------------------------------------------
+  // The slabs of all of this workgroup's tiles form one stream.  While slab r is multiplied, the B copies of slab
+  // r + 2 go straight to LDS (into the buffer of slab r, free after the barrier in the middle of the slab) and the A
+  // chunks of slab r + 3 are loaded into registers, from where the chunks of slab r + 1, loaded two slabs earlier,
+  // have just been written to LDS: A is the operand that comes from memory, B panels are shared through L2.
+  // Each of the two cursors holds the window (buffer descriptor) of the tile it is in and its offset along K.
+  struct Win { i32x4_t ra, rb; };
+  auto window = [&](const Tile& t, bool live) __attribute__((always_inline))  {
+    Win w;
+    const int n_left = p.N - t.n0;
+    w.ra = make_rsrc32((uint64_t)p.A + (uint64_t)(t.row0 * ld), live ? t.rows * ld : 0);  // only the tile's valid rows
+    w.rb = make_rsrc32((uint64_t)p.B + (uint64_t)(((int64_t)t.g * p.N + t.n0) * ld), live ? (n_left < C::BN ? n_left : C::BN) * ld : 0);
+    return w;
   };
   const TileWalk walk64 = sched_walk(num_tiles, p.tile_split != 0);
   struct { int first, end, stride; } walk = {(int)walk64.first, (int)walk64.end, (int)walk64.stride};
-  TileIo feed;
-  int feed_id;
-  Tile seen;
-  int seen_id = -1, seen_g = -1;
-  auto feed_seek = [&](int id) {
-    feed.kt_n = 0;
-    feed.issued = 0;
-    feed.a_base = feed.b_base = (uint64_t)p.A;
-    feed.a_rem = feed.b_rem = feed.b_off = 0;
-    if (id < walk.end) {
-      seen = sched_tile<C::BM, C::BN>(p, sched, id, seen_g);
-      seen_id = id;
-      seen_g = seen.g;
-      feed = make_io(seen);
-    }
-    feed_id = id;
+  const int row_bytes = __builtin_amdgcn_readfirstlane(ld);
+  int hint_g = -1;
+  auto tile_at = [&](int id, Tile& t) __attribute__((always_inline))  {  // false: the walk has ended
+    if (id >= walk.end) { t.g = 0; t.row0 = 0; t.rows = 0; t.n0 = 0; t.k0 = t.k1 = 0; return false; }
+    const Tile v = sched_tile<C::BM, C::BN>(p, sched, id, hint_g);
+    // the same in every lane; in scalar registers, so that what depends on it branches as a wave
+    t.g = __builtin_amdgcn_readfirstlane(v.g);
+    t.row0 = (int64_t)uniform64((uint64_t)v.row0);
+    t.rows = __builtin_amdgcn_readfirstlane(v.rows);
+    t.n0 = __builtin_amdgcn_readfirstlane(v.n0);
+    t.k0 = t.k1 = 0;
+    hint_g = t.g;
+    return true;
   };
-  struct SlabCopy {
-    i32x4_t ra, rb;
-    uint32_t base;
-    bool tail;
+
+  // The staged A chunks live in v[192:255] (two sets of eight), named in the instruction text: a value that is in
+  // flight across loop iterations must not be known to the compiler, which would move it between registers (before
+  // it has arrived) wherever two paths join.  The compiler's own allocation ends below v192 (checked on the kept
+  // assembly by the tests).
+#define TGG_W4_GA(c, f) \
+  if (c == 0) { f("224", "227") } else if (c == 1) { f("228", "231") } else if (c == 2) { f("232", "235") } else if (c == 3) { f("236", "239") } \
+  else if (c == 4) { f("240", "243") } else if (c == 5) { f("244", "247") } else if (c == 6) { f("248", "251") } else if (c == 7) { f("252", "255") } \
+  else if (c == 8) { f("192", "195") } else if (c == 9) { f("196", "199") } else if (c == 10) { f("200", "203") } else if (c == 11) { f("204", "207") } \
+  else if (c == 12) { f("208", "211") } else if (c == 13) { f("212", "215") } else if (c == 14) { f("216", "219") } else { f("220", "223") }
+#define TGG_W4_GA_CLOBBER "v192", "v193", "v194", "v195", "v196", "v197", "v198", "v199", "v200", "v201", "v202", "v203", "v204", "v205", "v206", "v207", \
+  "v208", "v209", "v210", "v211", "v212", "v213", "v214", "v215", "v216", "v217", "v218", "v219", "v220", "v221", "v222", "v223", "v224", "v225", "v226", "v227", \
+  "v228", "v229", "v230", "v231", "v232", "v233", "v234", "v235", "v236", "v237", "v238", "v239", "v240", "v241", "v242", "v243", "v244", "v245", "v246", "v247", \
+  "v248", "v249", "v250", "v251", "v252", "v253", "v254", "v255"
+  const uint32_t a_wr = smem_addr + wave * 1024 + lane * 16;  // LDS address of this lane's 16 bytes of A copy 0 (buffer 0)
+  // A chunk k of the slab at offset koff of window ra -> register set SET
+  auto load_a = [&](auto Kc, auto SETc, const i32x4_t& ra, int koff) __attribute__((always_inline))  {
+    constexpr int k = decltype(Kc)::value, kq = k + 8 * decltype(SETc)::value;
+    const int v = vo[k];
+#define TGG_W4_F(lo, hi) asm volatile("buffer_load_dwordx4 v[" lo ":" hi "], %0, %1, %2 offen" : : "v"(v), "s"(ra), "s"(koff) : "memory", TGG_W4_GA_CLOBBER);
+    TGG_W4_GA(kq, TGG_W4_F)
+#undef TGG_W4_F
   };
-  constexpr int CA = C::NI_A / C::NWAVES, CB = C::NI_B / C::NWAVES, NC = CA + CB;
-  static_assert(NC == 16, "one copy every fourth multiply of a K step");
-  auto begin_slab = [&](int buf) {
-    SlabCopy sc;
-    const bool live = feed.issued < feed.kt_n;
-    const int b_len = B_KMAJOR ? feed.b_rem : min(feed.b_rem, BK4) * b_ld - feed.b_off;
-    sc.ra = make_rsrc32(feed.a_base, live ? feed.a_rem : 0);
-    sc.rb = make_rsrc32(feed.b_base, live ? b_len : 0);
-    sc.base = smem_addr + buf * C::STAGE_BYTES;
-    sc.tail = tail_chunks != 0 && feed.issued + 1 == feed.kt_n;
-    feed.a_base += BK4 * 2;
-    feed.a_rem -= BK4 * 2;
-    feed.b_base += b_step;
-    feed.b_rem -= B_KMAJOR ? BK4 * 2 : BK4;
-    feed.issued += 1;
-    if (live && feed.issued >= feed.kt_n) feed_seek(feed_id + walk.stride);
-    return sc;
+  // register set SET, chunk k -> LDS (wr_addr: a_wr + the buffer's offset)
+  auto write_a = [&](auto Kc, auto SETc, uint32_t wr_addr) __attribute__((always_inline))  {
+    constexpr int k = decltype(Kc)::value, kq = k + 8 * decltype(SETc)::value;
+#define TGG_W4_F(lo, hi) asm volatile("ds_write_b128 %0, v[" lo ":" hi "] offset:%1" : : "v"(wr_addr), "n"(k * 4096) : "memory", TGG_W4_GA_CLOBBER);
+    TGG_W4_GA(kq, TGG_W4_F)
+#undef TGG_W4_F
   };
-  auto copy_k = [&](const SlabCopy& sc, int k) {  // k is a compile-time constant at every call site
-    if (k < CA) {
-      const int idx = wave + k * C::NWAVES;
-      copy_b128_to_lds(sc.ra, sc.base + idx * 1024, (sc.tail ? a_voff_tail[k & 1] : a_voff[k & 1]) + idx * OpA::RPI * a_ld);
-    } else {
-      const int kb = k - CA, idx = wave + kb * C::NWAVES;
-      copy_b128_to_lds(sc.rb, sc.base + C::A_BYTES + idx * 1024,
-                       (sc.tail ? b_voff_tail[kb & 1] : b_voff[kb & 1]) + idx * OpB::RPI * b_ld);
-    }
+  // B copy k of the slab at offset koff of window rb, straight to LDS, in two statements a multiply apart: the LDS
+  // address goes to m0 first (a copy to LDS needs a wait state after a write of m0; the multiply in between is one)
+  auto copy_b_m0 = [&](auto Kc, uint32_t buf_addr) __attribute__((always_inline))  {
+    constexpr int k = decltype(Kc)::value;
+    asm volatile("s_add_u32 m0, %0, %1" : : "s"(buf_addr), "n"(C::A_BYTES + 4 * k * 1024) : "memory", "m0", "scc");
   };
+  auto copy_b = [&](auto Kc, const i32x4_t& rb, int koff, bool spaced) __attribute__((always_inline))  {
+    constexpr int k = decltype(Kc)::value;
+    const int v = vo[k];
+    if (spaced) asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(v), "s"(rb), "s"(koff) : "memory");
+    else asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(v), "s"(rb), "s"(koff) : "memory");
+  };
+  // a slab's A copy k straight to LDS (prologue only)
+  auto copy_a_direct = [&](auto Kc, const i32x4_t& ra, int koff, uint32_t buf_addr) __attribute__((always_inline))  {
+    constexpr int k = decltype(Kc)::value;
+    const int v = vo[k];
+    asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %3, %4 offen lds"
+                 : : "s"(buf_addr), "n"(4 * k * 1024), "v"(v), "s"(ra), "s"(koff) : "memory", "m0", "scc");
+  };
+  const uint32_t wave_buf = smem_addr + wave * 1024;  // copy `wave` of buffer 0's A slab
 
   // ---- fragments and accumulators --------------------------------------------------------------------------------
   i32x4_t fa[2][8], fb[2][8];
@@ -221,18 +210,9 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   // (the next step needs all of them at once), then A fragments in the order of use
   auto read_frag = [&](auto KSc, auto Qc, i32x4_t (&sa)[8], i32x4_t (&sb)[8], uint32_t buf_off) {
     constexpr int KS = decltype(KSc)::value, Q = decltype(Qc)::value;
-    if (Q < 8) {
-      if (B_KMAJOR) lds_read_b128<Q * 2048>(sb[Q], b_rd[B_KMAJOR ? KS : 0] + buf_off);
-      else lds_read_tr<KS * 32 * (C::BN * 2), KS * 32 * (C::BN * 2) + 4 * (C::BN * 2)>(sb[Q], b_rd[B_KMAJOR ? 0 : Q] + buf_off);
-    } else {
-      lds_read_b128<(Q - 8) * 2048>(sa[Q - 8], a_rd[KS] + buf_off);
-    }
+    if (Q < 8) lds_read_b128<Q * 2048>(sb[Q], b_rd[KS] + buf_off);
+    else lds_read_b128<(Q - 8) * 2048>(sa[Q - 8], a_rd[KS] + buf_off);
   };
-  // One K step: 64 multiplies on set CUR (when MUL); the 16 fragments of K step NKS of the slab at nb_off go to the
-  // other set; when COPY, this wave's 16 copies of `sc` go out.
-  // Ends with the wait for those reads (and, when COPY is false, i.e. in front of the barrier, for this wave's copies
-  // of the next slab): the registers the reads target pass through the wait statement, inside the same straight-line
-  // code, before anything else may touch them.
   // ---- deferred epilogue ---------------------------------------------------------------------------------------------
   // A tile's results are stored during the first K step of the workgroup's next tile: with one wave per SIMD nothing
   // else would keep the matrix pipe busy while a wave converts and stores its 128x128 block.  A lane owns row l16 and
@@ -249,7 +229,7 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   char* const stage = smem + C::EPI_OFF + wave * C::EPI_WAVE_BYTES;
   // per-lane staging addresses and output offset, recomputed where a first K step or a flush begins
   struct EpiLane { char* wr; const char* rd; int off; int ch8; };
-  auto epi_lane = [&]() {
+  auto epi_lane = [&]() __attribute__((always_inline))  {
     int el = lane;
     asm volatile("" : "+v"(el));
     EpiLane e;
@@ -260,7 +240,7 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
     return e;
   };
   // block (i, j) -> staging piece j / 4; not before this point in the instruction stream
-  auto epi_cvt = [&](const EpiLane& e, int i, int j) {
+  auto epi_cvt = [&](const EpiLane& e, int i, int j) __attribute__((always_inline))  {
     asm volatile("" : "+a"(acc[i][j]));
     *(uint2*)(e.wr + (j >> 2) * C::EPI_PIECE + (j & 3) * 32) = pack4<DT>(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
     asm volatile("" ::: "memory");
@@ -270,7 +250,7 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
     for (int it = 0; it < 2; ++it) v[it] = *(const i32x4_t*)(e.rd + h * C::EPI_PIECE + it * 8 * C::EPI_PITCH);
     asm volatile("" ::: "memory");
   };
-  auto epi_store = [&](const EpiLane& e, int i, int h, int it, const i32x4_t& v) {
+  auto epi_store = [&](const EpiLane& e, int i, int h, int it, const i32x4_t& v) __attribute__((always_inline))  {
     const int off = (64 * h + e.ch8 < pend_cols) ? e.off + ((16 * i + 8 * it) * p.N + 64 * h) * 2 : kNoFetch;
     i32x4_t rs;
 #pragma unroll
@@ -280,7 +260,7 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
     asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, 0 offen nt\n\ts_nop 1" : : "v"(v), "v"(off), "s"(rs) : "memory");
   };
   // everything that is pending, without multiplies to hide it under
-  auto epi_flush = [&]() {
+  auto epi_flush = [&]() __attribute__((always_inline))  {
     if (pending) {
       // the last row block's multiplies may have just been issued: give them time before compiled code reads the registers
       asm volatile("s_nop 15\n\ts_nop 7" : "+a"(acc[7][0]), "+a"(acc[7][1]), "+a"(acc[7][2]), "+a"(acc[7][3]),
@@ -303,10 +283,46 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
     pend_rs[2] = 0;
   };
 
+
+  typedef std::integral_constant<int, 0> I0;
+  typedef std::integral_constant<int, 1> I1;
+  typedef std::integral_constant<int, 2> I2;
+  typedef std::integral_constant<bool, true> Yes;
+  typedef std::integral_constant<bool, false> No;
+
+  // the two cursors of the copy stream and the tile after the one being multiplied
+  i32x4_t ra_c, rb_c;
+  int koff_a, koff_b;
+  Win nxt;
+  Tile nxt_tile;
+  const int k_bytes = row_bytes;  // a tile's extent along K in bytes: where a cursor moves on to the next tile
+  auto advance_a = [&]() __attribute__((always_inline))  {
+    const bool wrap = koff_a + 128 == k_bytes;
+    koff_a = wrap ? 0 : koff_a + 128;
+#pragma unroll
+    for (int q = 0; q < 3; ++q) ra_c[q] = wrap ? nxt.ra[q] : ra_c[q];
+  };
+  auto advance_b = [&]() __attribute__((always_inline))  {
+    const bool wrap = koff_b + 128 == k_bytes;
+    koff_b = wrap ? 0 : koff_b + 128;
+#pragma unroll
+    for (int q = 0; q < 3; ++q) rb_c[q] = wrap ? nxt.rb[q] : rb_c[q];
+  };
+
+  // One K step: 64 multiplies on fragment set CUR (when MUL); the 16 fragments of K step NKS of the slab at nb_off go
+  // to the other set, one read every third multiply.  At most two other instructions sit between two multiplies: a
+  // wave issues in order, and what exceeds the sixteen cycles of a multiply leaves the matrix pipe idle.
+  // ROLE 0: prologue (reads only, waits for everything).
+  // ROLE 1: a slab's first K step.  The A chunks of the next slab go from register set SET to LDS (wr_addr) and the
+  //         chunks of the slab three ahead are requested into the same set; ends with the wait for the B copies of
+  //         the next slab (eight younger loads, and 32 stores in a tile's first K step, may stay in flight; loads
+  //         and stores complete in order, so the A chunks written here -- requested two slabs ago -- have arrived
+  //         since the previous such wait).
+  // ROLE 2: second K step: the B copies of the slab two ahead, into the buffer at cp_addr.
   // EPI: the first K step of a tile -- multiplies start from zero, and the pending epilogue runs between them.
-  auto kstep = [&](auto CURc, auto NKSc, auto MULc, auto COPYc, uint32_t nb_off, const SlabCopy& sc, auto EPIc) {
-    constexpr int CUR = decltype(CURc)::value, NKS = decltype(NKSc)::value;
-    constexpr bool MUL = decltype(MULc)::value, COPY = decltype(COPYc)::value, EPI = decltype(EPIc)::value;
+  auto kstep = [&](auto CURc, auto NKSc, auto MULc, auto ROLEc, uint32_t nb_off, auto EPIc, uint32_t wr_addr, auto SETc, uint32_t cp_addr) __attribute__((always_inline))  {
+    constexpr int CUR = decltype(CURc)::value, NKS = decltype(NKSc)::value, ROLE = decltype(ROLEc)::value;
+    constexpr bool MUL = decltype(MULc)::value, EPI = decltype(EPIc)::value;
     static_assert(!EPI || MUL, "the deferred epilogue rides on a multiplying K step");
     EpiLane e = {nullptr, nullptr, 0, 0};
     i32x4_t v0[2], v1[2];
@@ -337,68 +353,98 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
         TGG_W4_RD(0) TGG_W4_RD(1) TGG_W4_RD(2) TGG_W4_RD(3) TGG_W4_RD(4) TGG_W4_RD(5) TGG_W4_RD(6) TGG_W4_RD(7)
         TGG_W4_RD(8) TGG_W4_RD(9) TGG_W4_RD(10) TGG_W4_RD(11) TGG_W4_RD(12) TGG_W4_RD(13) TGG_W4_RD(14) TGG_W4_RD(15)
 #undef TGG_W4_RD
-        if (COPY && (n + 1) % 4 == 0) {
-          copy_k(sc, (n + 1) / 4 - 1);
-          if (!MUL) __builtin_amdgcn_s_sleep(1);  // a wave without multiplies must not crowd the address unit's queue
+        if (ROLE == 1) {
+#define TGG_W4_ST(c) if (n == 6 * c + 1) write_a(std::integral_constant<int, c>(), SETc, wr_addr); \
+                     if (n == 6 * c + 4) { load_a(std::integral_constant<int, c>(), SETc, ra_c, koff_a); if (!MUL) __builtin_amdgcn_s_sleep(1); }
+          TGG_W4_ST(0) TGG_W4_ST(1) TGG_W4_ST(2) TGG_W4_ST(3) TGG_W4_ST(4) TGG_W4_ST(5) TGG_W4_ST(6) TGG_W4_ST(7)
+#undef TGG_W4_ST
+          if (n == 52) advance_a();
+        }
+        if (ROLE == 2) {
+#define TGG_W4_CP(c) if (n == 6 * c + 3) copy_b_m0(std::integral_constant<int, c>(), cp_addr); \
+                     if (n == 6 * c + 4) { copy_b(std::integral_constant<int, c>(), rb_c, koff_b, MUL); if (!MUL) __builtin_amdgcn_s_sleep(1); }
+          TGG_W4_CP(0) TGG_W4_CP(1) TGG_W4_CP(2) TGG_W4_CP(3) TGG_W4_CP(4) TGG_W4_CP(5) TGG_W4_CP(6) TGG_W4_CP(7)
+#undef TGG_W4_CP
+          if (n == 52) advance_b();
         }
       }
-    if (COPY) asm volatile("s_waitcnt lgkmcnt(0)" : TGG_TIE8(fa[CUR ^ 1]), TGG_TIE8(fb[CUR ^ 1]) : : "memory");
+    if (ROLE == 2) asm volatile("s_waitcnt lgkmcnt(0)" : TGG_TIE8(fa[CUR ^ 1]), TGG_TIE8(fb[CUR ^ 1]) : : "memory");
+    else if (ROLE == 1) asm volatile("s_waitcnt vmcnt(%16) lgkmcnt(0)" : TGG_TIE8(fa[CUR ^ 1]), TGG_TIE8(fb[CUR ^ 1]) : "n"(EPI ? 40 : 8) : "memory");
     else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : TGG_TIE8(fa[CUR ^ 1]), TGG_TIE8(fb[CUR ^ 1]) : : "memory");
   };
-  typedef std::integral_constant<int, 0> I0;
-  typedef std::integral_constant<int, 1> I1;
-  typedef std::integral_constant<bool, true> Yes;
-  typedef std::integral_constant<bool, false> No;
 
-  // ---- prologue: slab 0 lands, its first fragments are read, slab 1 is requested -------------------------------------
-  feed_seek(walk.first);
+  // ---- prologue: slab 0 lands in buffer 0, slabs 1 and 2 are requested, the first fragments are read -----------------
+  Tile cur;
+  tile_at(walk.first, cur);
   {
-    const SlabCopy s0 = begin_slab(0);
-#pragma unroll
-    for (int k = 0; k < NC; ++k) copy_k(s0, k);
+    const Win w0 = window(cur, walk.first < walk.end);
+    const bool more = tile_at(walk.first + walk.stride, nxt_tile);
+    nxt = window(nxt_tile, more);
+    ra_c = w0.ra;
+    rb_c = w0.rb;
   }
+#define TGG_W4_EACH(f) f(0) f(1) f(2) f(3) f(4) f(5) f(6) f(7)
+#define TGG_W4_P0(c) copy_a_direct(std::integral_constant<int, c>(), ra_c, 0, wave_buf); \
+                     copy_a_direct(std::integral_constant<int, c>(), rb_c, 0, wave_buf + C::A_BYTES);
+  TGG_W4_EACH(TGG_W4_P0)
+#undef TGG_W4_P0
   wait_vmcnt<0>();
   __syncthreads();
-  {
-    const SlabCopy s1 = begin_slab(1);
-#pragma unroll
-    for (int k = 0; k < NC; ++k) copy_k(s1, k);
-  }
-  {
-    SlabCopy none;
-    kstep(I1(), I0(), No(), No(), 0u, none, No());  // reads K step 0 of buffer 0 into set 0, multiplies nothing, waits for everything
-  }
-  int ring = 0;
+#define TGG_W4_P1(c) load_a(std::integral_constant<int, c>(), I1(), ra_c, 128);
+  TGG_W4_EACH(TGG_W4_P1)
+#undef TGG_W4_P1
+#define TGG_W4_P2(c) copy_a_direct(std::integral_constant<int, c>(), rb_c, 128, wave_buf + C::STAGE_BYTES + C::A_BYTES);
+  TGG_W4_EACH(TGG_W4_P2)
+#undef TGG_W4_P2
+#define TGG_W4_P3(c) load_a(std::integral_constant<int, c>(), I0(), ra_c, 256);
+  TGG_W4_EACH(TGG_W4_P3)
+#undef TGG_W4_P3
+  koff_a = 3 * 128;  // at least four slabs per tile (w4_supported): both cursors are still in the first tile
+  koff_b = 2 * 128;
+  kstep(I1(), I0(), No(), I0(), 0u, No(), 0u, I0(), 0u);  // reads K step 0 of buffer 0 into set 0, multiplies nothing, waits for everything
+  const int kt_all = p.K / BK4;
 
   for (int tile_id = walk.first; tile_id < walk.end; tile_id += walk.stride) {
-    const Tile cur = tile_id == seen_id ? seen : sched_tile<C::BM, C::BN>(p, sched, tile_id);
     // a wave whose block of the tile has no rows or no columns multiplies nothing and stores nothing
     const bool active = wm0 < cur.rows && cur.n0 + wn0 < p.N;
+    // one slab; FIRST: the tile's first, whose first K step starts the accumulators afresh and carries the epilogue;
+    // PAR: parity of the slab = its LDS buffer; the A chunks of the next slab wait in register set 1 - PAR
     if (!active) epi_flush();  // no multiplies in this tile to hide the pending stores under
-    // one slab; FIRST: the tile's first, whose first K step starts the accumulators afresh and carries the epilogue
-    auto slab = [&](auto FIRST) {
-      const uint32_t cur_off = (ring & 1) * C::STAGE_BYTES, nxt_off = C::STAGE_BYTES - cur_off;
-      const SlabCopy sc = begin_slab(ring & 1);  // descriptors of the slab after the next one, into the current slab's buffer
-      if (active) kstep(I0(), I1(), Yes(), No(), cur_off, sc, FIRST);
-      else kstep(I0(), I1(), No(), No(), cur_off, sc, No());
+    auto slab = [&](auto FIRST, auto PARc) __attribute__((always_inline)) {
+      constexpr int PAR = decltype(PARc)::value;
+      typedef std::integral_constant<int, 1 - PAR> SetN;
+      constexpr uint32_t cur_off = PAR * C::STAGE_BYTES, nxt_off = C::STAGE_BYTES - cur_off;
+      if (active) kstep(I0(), I1(), Yes(), I1(), cur_off, FIRST, a_wr + nxt_off, SetN(), 0u);
+      else kstep(I0(), I1(), No(), I1(), cur_off, No(), a_wr + nxt_off, SetN(), 0u);
       // set 1 is complete, this wave has read all it needs of the current slab, its copies of the next slab have landed
       asm volatile("s_barrier" ::: "memory");
-      if (active) kstep(I1(), I0(), Yes(), Yes(), nxt_off, sc, No());
-      else kstep(I1(), I0(), No(), Yes(), nxt_off, sc, No());
-      ++ring;
+      if (active) kstep(I1(), I0(), Yes(), I2(), nxt_off, No(), 0u, I0(), wave_buf + cur_off);
+      else kstep(I1(), I0(), No(), I2(), nxt_off, No(), 0u, I0(), wave_buf + cur_off);
     };
-    slab(Yes());
-    for (int kt = 1; kt < kt_all; ++kt) slab(No());
-    if (!active) continue;
-    // what the next tile's first K step (or a flush) will store
-    const int rows_left = cur.rows - wm0;
-    pend_rs = make_rsrc32((uint64_t)p.C + (uint64_t)(((cur.row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2),
-                          (rows_left < 128 ? rows_left : 128) * p.N * 2);
-    pend_cols = __builtin_amdgcn_readfirstlane(p.N - cur.n0 - wn0);
-    pending = true;
+    slab(Yes(), I0());  // an even number of slabs per tile: every tile starts in buffer 0
+    slab(No(), I1());
+    for (int kt = 2; kt < kt_all; kt += 2) {
+      slab(No(), I0());
+      slab(No(), I1());
+    }
+    if (active) {
+      // what the next tile's first K step (or a flush) will store
+      const int rows_left = cur.rows - wm0;
+      pend_rs = make_rsrc32((uint64_t)p.C + (uint64_t)(((cur.row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2),
+                            (rows_left < 128 ? rows_left : 128) * p.N * 2);
+      pend_cols = __builtin_amdgcn_readfirstlane(p.N - cur.n0 - wn0);
+      pending = true;
+    }
+    // both cursors are in the next tile by now: it becomes the current one, and the one after it is looked up
+    cur = nxt_tile;
+    const bool more = tile_at(tile_id + 2 * walk.stride, nxt_tile);
+    nxt = window(nxt_tile, more);
   }
   epi_flush();
   wait_vmcnt<0>();  // trailing zero-length copies still write LDS
+#undef TGG_W4_EACH
+#undef TGG_W4_GA
+#undef TGG_W4_GA_CLOBBER
 }
 
 template <int DT, int LAYOUT>
@@ -431,12 +477,14 @@ bool w4_supported(const GemmParams& p, int dt, int layout, bool any_size) {
   if (p.q_fmt != 0 || p.G > kFastMaxGroups) return false;
   if ((p.N & 7) != 0 || p.K < 8 || (p.K & 7) != 0) return false;
   if ((int64_t)p.K * 2 * 256 >= (1ll << 30)) return false;
+  if (p.K % 128 != 0 || p.K < 256) return false;  // an even number of 64-deep slabs per tile, four at least
   if (any_size) return true;
   int grid = num_cus();
   if (p.grid_limit > 0 && p.grid_limit < grid) grid = p.grid_limit;
   const int64_t row_tiles = (p.m_total + 255) / 256;
   const int64_t narrow_tiles = row_tiles * ((p.N + 127) / 128);
-  return narrow_tiles > 4 * (int64_t)grid;
+  // groups of 512 rows and more on average: where the eight-wave kernels would choose 256-row tiles as well
+  return narrow_tiles > 4 * (int64_t)grid && p.m_total >= 512 * (int64_t)p.G;
 }
 
 int launch_w4_16bit(const GemmParams& p, int dt, int layout, hipStream_t s) {
