@@ -333,6 +333,40 @@ def test_masked_decode_sized_counts(dev):
         assert bool((out[g, mm:] == -5.0).all()), f"group {g}: rows beyond masked_m were written"
 
 
+@pytest.mark.parametrize("counts", ["large", "small", "mixed"])
+def test_masked_launch_that_both_kernels_look_at(dev, counts):
+    """A masked launch large enough for the four-wave kernel (K a multiple of 128, many tiles): it and the eight-wave
+    kernel are both enqueued and decide from the counts, on the device, which of them runs -- the four-wave kernel
+    where 256-row tiles pay (large counts), the eight-wave kernels otherwise (small counts: 128-row tiles).  Exact on
+    integer inputs in every regime, rows beyond masked_m untouched, and the same bits when either kernel is forced."""
+    G, m_max, N, K = 72, 512, 1032, 256
+    if counts == "large":
+        masked = [512 - (37 * g) % 200 for g in range(G)]
+    elif counts == "small":
+        masked = [(53 * g) % 100 for g in range(G)]
+    else:
+        masked = [(131 * g) % 513 for g in range(G)]
+    masked[5], masked[6] = 0, 512 if counts != "small" else 99
+    lhs = _ints((G * m_max, K), 31)
+    rhs = _ints((G, N, K), 32)
+    ref = torch.bmm(lhs.float().view(G, m_max, K), rhs.float().transpose(1, 2)).to(torch.bfloat16)
+    mm_dev = torch.tensor(masked, dtype=torch.int32, device=dev)
+    lhs_d, rhs_d = lhs.to(dev), rhs.to(dev)
+    outs = []
+    for four_wave in (1, 2, 0):  # decided on the device; four-wave kernel forced; eight-wave kernels only
+        _native.set_option("four_wave", four_wave)
+        try:
+            out = torch.full((G * m_max, N), -5.0, dtype=torch.bfloat16, device=dev)
+            m_grouped_gemm_masked(lhs_d, rhs_d, out, mm_dev, m_max)
+        finally:
+            _native.set_option("four_wave", 1)
+        outs.append(out.cpu().view(G, m_max, N))
+    for out in outs:
+        for g, mm in enumerate(masked):
+            assert torch.equal(out[g, :mm], ref[g, :mm]), f"group {g}"
+            assert bool((out[g, mm:] == -5.0).all()), f"group {g}: rows beyond masked_m were written"
+
+
 def test_masked_full_mask_reduces_to_bmm_exact(dev, variant):
     G, m_max, N, K = 4, 128, 128, 64
     lhs = _ints((G * m_max, K), 13)

@@ -176,7 +176,15 @@ static GemmParams params_fp8_block(const void* Aq, const float* sa, const void* 
 
 static int dispatch_16bit(const GemmParams& p, int dt, int layout, hipStream_t s) {
   const int force_generic = g_force_generic.load(), four_wave = g_four_wave.load();
-  if (!force_generic && four_wave && w4_supported(p, dt, layout, four_wave == 2)) return launch_w4_16bit(p, dt, layout, s);
+  if (!force_generic && four_wave && w4_supported(p, dt, layout, four_wave == 2)) {
+    if (p.mode != MODE_MASKED || four_wave == 2) return launch_w4_16bit(p, dt, layout, s);
+    // masked: whether 256-row tiles pay depends on the counts; both kernels look at them and exactly one runs
+    GemmParams q = p;
+    q.wide_gate = 1;
+    if (int e = launch_w4_16bit(q, dt, layout, s)) return e;
+    q.wide_gate = 2;
+    return launch_fast_16bit(q, dt, layout, s);
+  }
   if (!force_generic && fast_supported(p, dt, layout)) return launch_fast_16bit(p, dt, layout, s);
   return launch_generic_16bit(p, dt, layout, s);
 }

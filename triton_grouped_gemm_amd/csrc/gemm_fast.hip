@@ -722,6 +722,10 @@ __global__ __launch_bounds__(CW::THREADS) void gemm_fast_auto_kernel(const GemmP
     static_assert(CW::THREADS >= kFastMaxGroups && CS::BM * 2 == CW::BM, "sched_init's half-height prefix is CS's");
     stream = sched_short_tiles_pay<CW::BN>(p, sched);
   }
+  if constexpr (!std::is_void<CS>::value) {
+    // the four-wave kernel, launched in front of this one, has taken the launch (GemmParams::wide_gate)
+    if (p.wide_gate == 2 && sched_wide_tiles_chosen<CW::BM, CW::BN>(p, sched)) return;
+  }
   if (__builtin_expect(sched_num_tiles<CN::BM, CN::BN>(p, sched) > (int64_t)gridDim.x, 1)) {
     if constexpr (!std::is_void<CS>::value) {
       if (__builtin_expect(stream, 0)) {

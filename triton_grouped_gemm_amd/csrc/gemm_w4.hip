@@ -83,15 +83,22 @@ struct W4Cfg {
   static_assert(SMEM_BYTES <= 160 * 1024, "LDS budget");
 };
 
+// A is the operand that takes the long way through registers ("staged", s), B is copied straight to LDS ("direct",
+// d).  Staging B instead makes no difference even where the weights are what streams from memory (masked decode:
+// 0.526 ms either way).
 template <int DT, int LAYOUT>
 __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParams p) {
   typedef W4Cfg C;
+  constexpr int S_OFF = 0, D_OFF = C::A_BYTES;  // the operands' places in a slab buffer
   static_assert(LAYOUT == W4_NT, "both operands K-contiguous");
   typedef Operand<C::BM, true> Op;  // A and B slabs have the same geometry: 256 rows of 128 bytes
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::SCHED_OFF);
   sched_init<C::BM>(p, sched);
+  // a launch that only pays where the eight-wave kernels would choose 256x256 tiles as well (GemmParams::wide_gate):
+  // the same predicate on the same table decides there that the eight-wave launch behind this one has nothing to do
+  if (p.wide_gate == 1 && !sched_wide_tiles_chosen<C::BM, C::BN>(p, sched)) return;
   const int num_tiles = (int)sched_num_tiles<C::BM, C::BN>(p, sched);
 
   const uint32_t smem_addr = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
@@ -123,12 +130,12 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   // chunks of slab r + 3 are loaded into registers, from where the chunks of slab r + 1, loaded two slabs earlier,
   // have just been written to LDS: A is the operand that comes from memory, B panels are shared through L2.
   // Each of the two cursors holds the window (buffer descriptor) of the tile it is in and its offset along K.
-  struct Win { i32x4_t ra, rb; };
+  struct Win { i32x4_t rs, rd; };  // staged operand, directly copied operand
   auto window = [&](const Tile& t, bool live) __attribute__((always_inline))  {
     Win w;
     const int n_left = p.N - t.n0;
-    w.ra = make_rsrc32((uint64_t)p.A + (uint64_t)(t.row0 * ld), live ? t.rows * ld : 0);  // only the tile's valid rows
-    w.rb = make_rsrc32((uint64_t)p.B + (uint64_t)(((int64_t)t.g * p.N + t.n0) * ld), live ? (n_left < C::BN ? n_left : C::BN) * ld : 0);
+    w.rs = make_rsrc32((uint64_t)p.A + (uint64_t)(t.row0 * ld), live ? t.rows * ld : 0);  // only the tile's valid rows
+    w.rd = make_rsrc32((uint64_t)p.B + (uint64_t)(((int64_t)t.g * p.N + t.n0) * ld), live ? (n_left < C::BN ? n_left : C::BN) * ld : 0);
     return w;
   };
   const TileWalk walk64 = sched_walk(num_tiles, p.tile_split != 0);
@@ -161,17 +168,17 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   "v208", "v209", "v210", "v211", "v212", "v213", "v214", "v215", "v216", "v217", "v218", "v219", "v220", "v221", "v222", "v223", "v224", "v225", "v226", "v227", \
   "v228", "v229", "v230", "v231", "v232", "v233", "v234", "v235", "v236", "v237", "v238", "v239", "v240", "v241", "v242", "v243", "v244", "v245", "v246", "v247", \
   "v248", "v249", "v250", "v251", "v252", "v253", "v254", "v255"
-  const uint32_t a_wr = smem_addr + wave * 1024 + lane * 16;  // LDS address of this lane's 16 bytes of A copy 0 (buffer 0)
+  const uint32_t s_wr = smem_addr + S_OFF + wave * 1024 + lane * 16;  // LDS address of this lane's 16 bytes of A copy 0 (buffer 0)
   // A chunk k of the slab at offset koff of window ra -> register set SET
-  auto load_a = [&](auto Kc, auto SETc, const i32x4_t& ra, int koff) __attribute__((always_inline))  {
+  auto load_s = [&](auto Kc, auto SETc, const i32x4_t& ra, int koff) __attribute__((always_inline))  {
     constexpr int k = decltype(Kc)::value, kq = k + 8 * decltype(SETc)::value;
     const int v = vo[k];
 #define TGG_W4_F(lo, hi) asm volatile("buffer_load_dwordx4 v[" lo ":" hi "], %0, %1, %2 offen" : : "v"(v), "s"(ra), "s"(koff) : "memory", TGG_W4_GA_CLOBBER);
     TGG_W4_GA(kq, TGG_W4_F)
 #undef TGG_W4_F
   };
-  // register set SET, chunk k -> LDS (wr_addr: a_wr + the buffer's offset)
-  auto write_a = [&](auto Kc, auto SETc, uint32_t wr_addr) __attribute__((always_inline))  {
+  // register set SET, chunk k -> LDS (wr_addr: s_wr + the buffer's offset)
+  auto write_s = [&](auto Kc, auto SETc, uint32_t wr_addr) __attribute__((always_inline))  {
     constexpr int k = decltype(Kc)::value, kq = k + 8 * decltype(SETc)::value;
 #define TGG_W4_F(lo, hi) asm volatile("ds_write_b128 %0, v[" lo ":" hi "] offset:%1" : : "v"(wr_addr), "n"(k * 4096) : "memory", TGG_W4_GA_CLOBBER);
     TGG_W4_GA(kq, TGG_W4_F)
@@ -179,18 +186,18 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   };
   // B copy k of the slab at offset koff of window rb, straight to LDS, in two statements a multiply apart: the LDS
   // address goes to m0 first (a copy to LDS needs a wait state after a write of m0; the multiply in between is one)
-  auto copy_b_m0 = [&](auto Kc, uint32_t buf_addr) __attribute__((always_inline))  {
+  auto copy_d_m0 = [&](auto Kc, uint32_t buf_addr) __attribute__((always_inline))  {
     constexpr int k = decltype(Kc)::value;
-    asm volatile("s_add_u32 m0, %0, %1" : : "s"(buf_addr), "n"(C::A_BYTES + 4 * k * 1024) : "memory", "m0", "scc");
+    asm volatile("s_add_u32 m0, %0, %1" : : "s"(buf_addr), "n"(D_OFF + 4 * k * 1024) : "memory", "m0", "scc");
   };
-  auto copy_b = [&](auto Kc, const i32x4_t& rb, int koff, bool spaced) __attribute__((always_inline))  {
+  auto copy_d = [&](auto Kc, const i32x4_t& rb, int koff, bool spaced) __attribute__((always_inline))  {
     constexpr int k = decltype(Kc)::value;
     const int v = vo[k];
     if (spaced) asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(v), "s"(rb), "s"(koff) : "memory");
     else asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(v), "s"(rb), "s"(koff) : "memory");
   };
   // a slab's A copy k straight to LDS (prologue only)
-  auto copy_a_direct = [&](auto Kc, const i32x4_t& ra, int koff, uint32_t buf_addr) __attribute__((always_inline))  {
+  auto copy_direct = [&](auto Kc, const i32x4_t& ra, int koff, uint32_t buf_addr) __attribute__((always_inline))  {
     constexpr int k = decltype(Kc)::value;
     const int v = vo[k];
     asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %3, %4 offen lds"
@@ -291,22 +298,22 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   typedef std::integral_constant<bool, false> No;
 
   // the two cursors of the copy stream and the tile after the one being multiplied
-  i32x4_t ra_c, rb_c;
-  int koff_a, koff_b;
+  i32x4_t rs_c, rd_c;
+  int koff_s, koff_d;
   Win nxt;
   Tile nxt_tile;
   const int k_bytes = row_bytes;  // a tile's extent along K in bytes: where a cursor moves on to the next tile
-  auto advance_a = [&]() __attribute__((always_inline))  {
-    const bool wrap = koff_a + 128 == k_bytes;
-    koff_a = wrap ? 0 : koff_a + 128;
+  auto advance_s = [&]() __attribute__((always_inline))  {
+    const bool wrap = koff_s + 128 == k_bytes;
+    koff_s = wrap ? 0 : koff_s + 128;
 #pragma unroll
-    for (int q = 0; q < 3; ++q) ra_c[q] = wrap ? nxt.ra[q] : ra_c[q];
+    for (int q = 0; q < 3; ++q) rs_c[q] = wrap ? nxt.rs[q] : rs_c[q];
   };
-  auto advance_b = [&]() __attribute__((always_inline))  {
-    const bool wrap = koff_b + 128 == k_bytes;
-    koff_b = wrap ? 0 : koff_b + 128;
+  auto advance_d = [&]() __attribute__((always_inline))  {
+    const bool wrap = koff_d + 128 == k_bytes;
+    koff_d = wrap ? 0 : koff_d + 128;
 #pragma unroll
-    for (int q = 0; q < 3; ++q) rb_c[q] = wrap ? nxt.rb[q] : rb_c[q];
+    for (int q = 0; q < 3; ++q) rd_c[q] = wrap ? nxt.rd[q] : rd_c[q];
   };
 
   // One K step: 64 multiplies on fragment set CUR (when MUL); the 16 fragments of K step NKS of the slab at nb_off go
@@ -354,18 +361,18 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
         TGG_W4_RD(8) TGG_W4_RD(9) TGG_W4_RD(10) TGG_W4_RD(11) TGG_W4_RD(12) TGG_W4_RD(13) TGG_W4_RD(14) TGG_W4_RD(15)
 #undef TGG_W4_RD
         if (ROLE == 1) {
-#define TGG_W4_ST(c) if (n == 6 * c + 1) write_a(std::integral_constant<int, c>(), SETc, wr_addr); \
-                     if (n == 6 * c + 4) { load_a(std::integral_constant<int, c>(), SETc, ra_c, koff_a); if (!MUL) __builtin_amdgcn_s_sleep(1); }
+#define TGG_W4_ST(c) if (n == 6 * c + 1) write_s(std::integral_constant<int, c>(), SETc, wr_addr); \
+                     if (n == 6 * c + 4) { load_s(std::integral_constant<int, c>(), SETc, rs_c, koff_s); if (!MUL) __builtin_amdgcn_s_sleep(1); }
           TGG_W4_ST(0) TGG_W4_ST(1) TGG_W4_ST(2) TGG_W4_ST(3) TGG_W4_ST(4) TGG_W4_ST(5) TGG_W4_ST(6) TGG_W4_ST(7)
 #undef TGG_W4_ST
-          if (n == 52) advance_a();
+          if (n == 52) advance_s();
         }
         if (ROLE == 2) {
-#define TGG_W4_CP(c) if (n == 6 * c + 3) copy_b_m0(std::integral_constant<int, c>(), cp_addr); \
-                     if (n == 6 * c + 4) { copy_b(std::integral_constant<int, c>(), rb_c, koff_b, MUL); if (!MUL) __builtin_amdgcn_s_sleep(1); }
+#define TGG_W4_CP(c) if (n == 6 * c + 3) copy_d_m0(std::integral_constant<int, c>(), cp_addr); \
+                     if (n == 6 * c + 4) { copy_d(std::integral_constant<int, c>(), rd_c, koff_d, MUL); if (!MUL) __builtin_amdgcn_s_sleep(1); }
           TGG_W4_CP(0) TGG_W4_CP(1) TGG_W4_CP(2) TGG_W4_CP(3) TGG_W4_CP(4) TGG_W4_CP(5) TGG_W4_CP(6) TGG_W4_CP(7)
 #undef TGG_W4_CP
-          if (n == 52) advance_b();
+          if (n == 52) advance_d();
         }
       }
     if (ROLE == 2) asm volatile("s_waitcnt lgkmcnt(0)" : TGG_TIE8(fa[CUR ^ 1]), TGG_TIE8(fb[CUR ^ 1]) : : "memory");
@@ -380,27 +387,27 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
     const Win w0 = window(cur, walk.first < walk.end);
     const bool more = tile_at(walk.first + walk.stride, nxt_tile);
     nxt = window(nxt_tile, more);
-    ra_c = w0.ra;
-    rb_c = w0.rb;
+    rs_c = w0.rs;
+    rd_c = w0.rd;
   }
 #define TGG_W4_EACH(f) f(0) f(1) f(2) f(3) f(4) f(5) f(6) f(7)
-#define TGG_W4_P0(c) copy_a_direct(std::integral_constant<int, c>(), ra_c, 0, wave_buf); \
-                     copy_a_direct(std::integral_constant<int, c>(), rb_c, 0, wave_buf + C::A_BYTES);
+#define TGG_W4_P0(c) copy_direct(std::integral_constant<int, c>(), rs_c, 0, wave_buf + S_OFF); \
+                     copy_direct(std::integral_constant<int, c>(), rd_c, 0, wave_buf + D_OFF);
   TGG_W4_EACH(TGG_W4_P0)
 #undef TGG_W4_P0
   wait_vmcnt<0>();
   __syncthreads();
-#define TGG_W4_P1(c) load_a(std::integral_constant<int, c>(), I1(), ra_c, 128);
+#define TGG_W4_P1(c) load_s(std::integral_constant<int, c>(), I1(), rs_c, 128);
   TGG_W4_EACH(TGG_W4_P1)
 #undef TGG_W4_P1
-#define TGG_W4_P2(c) copy_a_direct(std::integral_constant<int, c>(), rb_c, 128, wave_buf + C::STAGE_BYTES + C::A_BYTES);
+#define TGG_W4_P2(c) copy_direct(std::integral_constant<int, c>(), rd_c, 128, wave_buf + C::STAGE_BYTES + D_OFF);
   TGG_W4_EACH(TGG_W4_P2)
 #undef TGG_W4_P2
-#define TGG_W4_P3(c) load_a(std::integral_constant<int, c>(), I0(), ra_c, 256);
+#define TGG_W4_P3(c) load_s(std::integral_constant<int, c>(), I0(), rs_c, 256);
   TGG_W4_EACH(TGG_W4_P3)
 #undef TGG_W4_P3
-  koff_a = 3 * 128;  // at least four slabs per tile (w4_supported): both cursors are still in the first tile
-  koff_b = 2 * 128;
+  koff_s = 3 * 128;  // at least four slabs per tile (w4_supported): both cursors are still in the first tile
+  koff_d = 2 * 128;
   kstep(I1(), I0(), No(), I0(), 0u, No(), 0u, I0(), 0u);  // reads K step 0 of buffer 0 into set 0, multiplies nothing, waits for everything
   const int kt_all = p.K / BK4;
 
@@ -414,8 +421,8 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
       constexpr int PAR = decltype(PARc)::value;
       typedef std::integral_constant<int, 1 - PAR> SetN;
       constexpr uint32_t cur_off = PAR * C::STAGE_BYTES, nxt_off = C::STAGE_BYTES - cur_off;
-      if (active) kstep(I0(), I1(), Yes(), I1(), cur_off, FIRST, a_wr + nxt_off, SetN(), 0u);
-      else kstep(I0(), I1(), No(), I1(), cur_off, No(), a_wr + nxt_off, SetN(), 0u);
+      if (active) kstep(I0(), I1(), Yes(), I1(), cur_off, FIRST, s_wr + nxt_off, SetN(), 0u);
+      else kstep(I0(), I1(), No(), I1(), cur_off, No(), s_wr + nxt_off, SetN(), 0u);
       // set 1 is complete, this wave has read all it needs of the current slab, its copies of the next slab have landed
       asm volatile("s_barrier" ::: "memory");
       if (active) kstep(I1(), I0(), Yes(), I2(), nxt_off, No(), 0u, I0(), wave_buf + cur_off);
@@ -473,7 +480,9 @@ int launch_w4(const GemmParams& p, hipStream_t s) {
 bool w4_supported(const GemmParams& p, int dt, int layout, bool any_size) {
   if (dt != DT_BF16 && dt != DT_F16) return false;
   if (layout != W4_NT) return false;
-  if (p.mode != MODE_MG && p.mode != MODE_MG_PAD) return false;
+  if (p.mode != MODE_MG && p.mode != MODE_MG_PAD && p.mode != MODE_MASKED) return false;
+  // masked launches are decided on the device, by a predicate that needs one thread of this kernel per group
+  if (p.mode == MODE_MASKED && p.G > W4Cfg::THREADS) return false;
   if (p.q_fmt != 0 || p.G > kFastMaxGroups) return false;
   if ((p.N & 7) != 0 || p.K < 8 || (p.K & 7) != 0) return false;
   if ((int64_t)p.K * 2 * 256 >= (1ll << 30)) return false;
@@ -484,7 +493,7 @@ bool w4_supported(const GemmParams& p, int dt, int layout, bool any_size) {
   const int64_t row_tiles = (p.m_total + 255) / 256;
   const int64_t narrow_tiles = row_tiles * ((p.N + 127) / 128);
   // groups of 512 rows and more on average: where the eight-wave kernels would choose 256-row tiles as well
-  return narrow_tiles > 4 * (int64_t)grid && p.m_total >= 512 * (int64_t)p.G;
+  return narrow_tiles > 4 * (int64_t)grid && (p.mode == MODE_MASKED || p.m_total >= 512 * (int64_t)p.G);
 }
 
 int launch_w4_16bit(const GemmParams& p, int dt, int layout, hipStream_t s) {

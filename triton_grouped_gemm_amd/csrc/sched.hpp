@@ -237,6 +237,14 @@ __device__ __forceinline__ bool sched_short_tiles_pay(const GemmParams& p, const
   return rounds_half * 7 <= rounds_full * 10;
 }
 
+// Whether a launch of 256-row tiles is neither small enough for the narrow tiles (all of them fit one round of the
+// persistent workgroups) nor made of groups so small that 128-row tiles pay: the case in which the eight-wave kernels
+// run their BM x BN configuration.  t: a table built by sched_init<BM> with one thread per group.
+template <int BM, int BN, class Table>
+__device__ __forceinline__ bool sched_wide_tiles_chosen(const GemmParams& p, const Table& t) {
+  return sched_num_tiles<BM, BN / 2>(p, t) > (int64_t)gridDim.x && !sched_short_tiles_pay<BN>(p, t);
+}
+
 // Tile order.  Consecutive tile ids are handed to workgroups that run at the same time on one XCD
 // (see sched_walk), so a run of ids should cover a near-square block of tiles: a run of R tiles spanning
 // w column tiles touches R / w row panels of A plus w column panels of B per K slab.  The N tiles are
