@@ -86,7 +86,11 @@ struct W4Cfg {
 // A is the operand that takes the long way through registers ("staged", s), B is copied straight to LDS ("direct",
 // d).  Staging B instead makes no difference even where the weights are what streams from memory (masked decode:
 // 0.526 ms either way).
-template <int DT, int LAYOUT>
+// SIT_OUT: a wave whose block of a tile has no rows or no columns multiplies nothing in that tile (it keeps its share
+// of the copy stream and the barriers going).  Worth 2 % where a quarter of the tiles have at most 128 rows (masked
+// decode); where nearly every tile is full the branch per K step costs the others 1 %, and such a wave multiplies
+// the zeros its windows deliver.
+template <int DT, int LAYOUT, bool SIT_OUT>
 __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParams p) {
   typedef W4Cfg C;
   constexpr int S_OFF = 0, D_OFF = C::A_BYTES;  // the operands' places in a slab buffer
@@ -412,20 +416,20 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   const int kt_all = p.K / BK4;
 
   for (int tile_id = walk.first; tile_id < walk.end; tile_id += walk.stride) {
-    // a wave whose block of the tile has no rows or no columns multiplies nothing and stores nothing
-    const bool active = wm0 < cur.rows && cur.n0 + wn0 < p.N;
+    const bool active = wm0 < cur.rows && cur.n0 + wn0 < p.N;  // this wave's block of the tile has rows and columns
+    const bool mul = !SIT_OUT || active;
+    if (!mul) epi_flush();  // no multiplies in this tile to hide the pending stores under
     // one slab; FIRST: the tile's first, whose first K step starts the accumulators afresh and carries the epilogue;
     // PAR: parity of the slab = its LDS buffer; the A chunks of the next slab wait in register set 1 - PAR
-    if (!active) epi_flush();  // no multiplies in this tile to hide the pending stores under
     auto slab = [&](auto FIRST, auto PARc) __attribute__((always_inline)) {
       constexpr int PAR = decltype(PARc)::value;
       typedef std::integral_constant<int, 1 - PAR> SetN;
       constexpr uint32_t cur_off = PAR * C::STAGE_BYTES, nxt_off = C::STAGE_BYTES - cur_off;
-      if (active) kstep(I0(), I1(), Yes(), I1(), cur_off, FIRST, s_wr + nxt_off, SetN(), 0u);
+      if (mul) kstep(I0(), I1(), Yes(), I1(), cur_off, FIRST, s_wr + nxt_off, SetN(), 0u);
       else kstep(I0(), I1(), No(), I1(), cur_off, No(), s_wr + nxt_off, SetN(), 0u);
       // set 1 is complete, this wave has read all it needs of the current slab, its copies of the next slab have landed
       asm volatile("s_barrier" ::: "memory");
-      if (active) kstep(I1(), I0(), Yes(), I2(), nxt_off, No(), 0u, I0(), wave_buf + cur_off);
+      if (mul) kstep(I1(), I0(), Yes(), I2(), nxt_off, No(), 0u, I0(), wave_buf + cur_off);
       else kstep(I1(), I0(), No(), I2(), nxt_off, No(), 0u, I0(), wave_buf + cur_off);
     };
     slab(Yes(), I0());  // an even number of slabs per tile: every tile starts in buffer 0
@@ -434,14 +438,13 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
       slab(No(), I0());
       slab(No(), I1());
     }
-    if (active) {
-      // what the next tile's first K step (or a flush) will store
-      const int rows_left = cur.rows - wm0;
-      pend_rs = make_rsrc32((uint64_t)p.C + (uint64_t)(((cur.row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2),
-                            (rows_left < 128 ? rows_left : 128) * p.N * 2);
-      pend_cols = __builtin_amdgcn_readfirstlane(p.N - cur.n0 - wn0);
-      pending = true;
-    }
+    // what the next tile's first K step (or the flush at the end) will store: nothing for a wave whose block of the
+    // tile has no rows or no columns
+    const int rows_left = cur.rows - wm0;
+    pend_rs = make_rsrc32((uint64_t)p.C + (uint64_t)(((cur.row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2),
+                          active ? (rows_left < 128 ? rows_left : 128) * p.N * 2 : 0);
+    pend_cols = __builtin_amdgcn_readfirstlane(active ? p.N - cur.n0 - wn0 : 0);
+    pending = mul;  // a wave that sat the tile out has flushed and left nothing behind
     // both cursors are in the next tile by now: it becomes the current one, and the one after it is looked up
     cur = nxt_tile;
     const bool more = tile_at(tile_id + 2 * walk.stride, nxt_tile);
@@ -454,13 +457,13 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
 #undef TGG_W4_GA_CLOBBER
 }
 
-template <int DT, int LAYOUT>
+template <int DT, int LAYOUT, bool SIT_OUT>
 int launch_w4(const GemmParams& p, hipStream_t s) {
   static bool attr_set[64] = {false};
   int dev = 0;
   (void)hipGetDevice(&dev);
   const bool listed = dev >= 0 && dev < 64;
-  auto kern = gemm_w4_kernel<DT, LAYOUT>;
+  auto kern = gemm_w4_kernel<DT, LAYOUT, SIT_OUT>;
   if (!listed || !attr_set[dev]) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, W4Cfg::SMEM_BYTES) != hipSuccess)
       return check_launch("hipFuncSetAttribute(gemm_w4)");
@@ -497,8 +500,9 @@ bool w4_supported(const GemmParams& p, int dt, int layout, bool any_size) {
 }
 
 int launch_w4_16bit(const GemmParams& p, int dt, int layout, hipStream_t s) {
-  if (dt == DT_BF16) return launch_w4<DT_BF16, W4_NT>(p, s);
-  return launch_w4<DT_F16, W4_NT>(p, s);
+  const bool sit_out = p.mode == MODE_MASKED;
+  if (dt == DT_BF16) return sit_out ? launch_w4<DT_BF16, W4_NT, true>(p, s) : launch_w4<DT_BF16, W4_NT, false>(p, s);
+  return sit_out ? launch_w4<DT_F16, W4_NT, true>(p, s) : launch_w4<DT_F16, W4_NT, false>(p, s);
 }
 
 }  // namespace tgg
