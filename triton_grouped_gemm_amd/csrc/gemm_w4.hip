@@ -29,8 +29,10 @@
 // accumulators.  That K step is the one place where a gap holds a dozen instructions (8 % of a launch).
 //
 // Headline shape (G = 128, M = 655360, N = 1536, K = 2048), same box: 3.18 ms against 3.30 ms for the eight-wave
-// kernel; K = 768 shape 1.91 against 1.97 ms.  Large launches with K a multiple of 128 take this kernel
-// (w4_supported), everything else the eight-wave kernels.
+// kernel; K = 768 shape 1.91 against 1.97 ms; masked decode (G = 128, up to 512 rows per group, N = 4096, K = 1536)
+// 0.53 against 0.56 ms.  Large M-grouped launches with K a multiple of 128 take this kernel (w4_supported); masked
+// launches of that size enqueue it together with the eight-wave kernel and the counts decide on the device which of
+// the two runs (GemmParams::wide_gate); everything else goes to the eight-wave kernels.
 //
 // What the compiler does not know about assembly statements, and how it is handled here:
 //   * a fragment read's result arrives later: every register a read targets passes through the wait statement
