@@ -73,35 +73,40 @@ def test_m_grouped_exact_on_integer_inputs(dev, variant, dtype, trans_b, sizes, 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("num_cu", [-1, 8, 3])  # few workgroups: each one's copy stream crosses many tile boundaries
-@pytest.mark.parametrize("sizes,N,K", [
-    ([300, 0, 417, 256, 1, 700], 520, 256),   # four slabs per tile, the least the four-wave kernel takes; a column tail of 8
-    ([129, 511, 0, 64], 1000, 384),
-    ([1024, 77], 256, 1024),
-    ([5, 0, 0, 250, 3], 136, 512),            # a single column tile whose right half lies beyond N: two waves sit every tile out
+@pytest.mark.parametrize("sizes,N,K,trans_b", [
+    ([300, 0, 417, 256, 1, 700], 520, 256, True),   # four slabs per tile, the least the four-wave kernel takes; a column tail of 8
+    ([129, 511, 0, 64], 1000, 384, True),
+    ([1024, 77], 256, 1024, True),
+    ([5, 0, 0, 250, 3], 136, 512, True),            # a single column tile whose right half lies beyond N
+    ([300, 0, 417, 256, 1, 700], 512, 256, False),  # B as [G, K, N]: N a multiple of 256
+    ([129, 511, 0, 64], 1024, 384, False),
+    ([1024, 77], 256, 1024, False),
 ])
-def test_four_wave_kernel_on_the_shapes_it_takes(dev, dtype, num_cu, sizes, N, K):
-    """K a multiple of 128 and at least 256: the four-wave kernel, forced, runs these itself (other K fall back to the
-    eight-wave kernels, which is what the `four_wave` variant of the other tests exercises).  Integer inputs against
-    the oracle bit for bit, then random inputs against the shape-agnostic kernel bit for bit."""
+def test_four_wave_kernel_on_the_shapes_it_takes(dev, dtype, num_cu, sizes, N, K, trans_b):
+    """K a multiple of 128 and at least 256 (and, with B as [G, K, N], N a multiple of 256): the four-wave kernel,
+    forced, runs these itself (other shapes fall back to the eight-wave kernels, which is what the `four_wave`
+    variant of the other tests exercises).  Integer inputs against the oracle bit for bit, then random inputs against
+    the shape-agnostic kernel bit for bit."""
     M = sum(sizes)
     s = torch.tensor(sizes, dtype=torch.int32, device=dev)
-    a_i, b_i = _ints((M, K), 3, dtype), _ints((len(sizes), N, K), 4, dtype)
+    b_shape = (len(sizes), N, K) if trans_b else (len(sizes), K, N)
+    a_i, b_i = _ints((M, K), 3, dtype), _ints(b_shape, 4, dtype)
     torch.manual_seed(K + N)
     a_r = (torch.randn(M, K, device=dev) * K ** -0.5).to(dtype)
-    b_r = torch.randn(len(sizes), N, K, device=dev).to(dtype)
+    b_r = torch.randn(b_shape, device=dev).to(dtype)
     _native.set_option("force_generic", 1)
     try:
-        ref_r = m_grouped_gemm(a_r, b_r, s, True)
+        ref_r = m_grouped_gemm(a_r, b_r, s, trans_b)
     finally:
         _native.set_option("force_generic", 0)
     _native.set_option("four_wave", 2)
     try:
-        out_i = m_grouped_gemm(a_i.to(dev), b_i.to(dev), s, True, numSM=num_cu)
-        out_r = m_grouped_gemm(a_r, b_r, s, True, numSM=num_cu)
-        out_r2 = m_grouped_gemm(a_r, b_r, s, True, numSM=num_cu)
+        out_i = m_grouped_gemm(a_i.to(dev), b_i.to(dev), s, trans_b, numSM=num_cu)
+        out_r = m_grouped_gemm(a_r, b_r, s, trans_b, numSM=num_cu)
+        out_r2 = m_grouped_gemm(a_r, b_r, s, trans_b, numSM=num_cu)
     finally:
         _native.set_option("four_wave", 1)
-    assert torch.equal(out_i.cpu(), gemm_ref.gmm_fp32(a_i, b_i, sizes, True).to(dtype))
+    assert torch.equal(out_i.cpu(), gemm_ref.gmm_fp32(a_i, b_i, sizes, trans_b).to(dtype))
     assert torch.equal(out_r, ref_r) and torch.equal(out_r2, ref_r)
 
 

@@ -51,7 +51,7 @@ namespace tgg {
 
 namespace {
 
-enum : int { W4_NT = 0 };
+enum : int { W4_NT = 0, W4_NN = 1 };
 constexpr int BK4 = 64;
 
 template <int DT> TGG_DEV void mfma_acc(f32x4_t& acc, const i32x4_t& w, const i32x4_t& x) {
@@ -68,6 +68,13 @@ template <int DT> TGG_DEV void mfma_new(f32x4_t& acc, const i32x4_t& w, const i3
 // 16-byte fragment of a K-contiguous operand
 template <int OFF> TGG_DEV void lds_read_b128(i32x4_t& dst, uint32_t addr) {
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
+// fragment of a token-row operand: two transposing 8-byte reads (K 0..3 and 4..7 of the lane's column)
+template <int OFF0, int OFF1> TGG_DEV void lds_read_tr(i32x4_t& dst, uint32_t addr) {
+  i32x2_t lo, hi;
+  asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+               : "=&v"(lo), "=&v"(hi) : "v"(addr), "n"(OFF0), "n"(OFF1) : "memory");
+  dst = __builtin_shufflevector(lo, hi, 0, 1, 2, 3);
 }
 #define TGG_TIE8(f) "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]), "+v"(f[6]), "+v"(f[7])
 
@@ -96,8 +103,9 @@ template <int DT, int LAYOUT, bool SIT_OUT>
 __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParams p) {
   typedef W4Cfg C;
   constexpr int S_OFF = 0, D_OFF = C::A_BYTES;  // the operands' places in a slab buffer
-  static_assert(LAYOUT == W4_NT, "both operands K-contiguous");
-  typedef Operand<C::BM, true> Op;  // A and B slabs have the same geometry: 256 rows of 128 bytes
+  constexpr bool B_KMAJOR = LAYOUT == W4_NT;  // NN: B is [G, K, N], its slab 64 token rows of 512 bytes (N a multiple of 256)
+  typedef Operand<C::BM, true> Op;            // the A slab, and B's when K-contiguous: 256 rows of 128 bytes
+  typedef Operand<C::BN, B_KMAJOR> OpB;
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   auto& sched = *reinterpret_cast<SchedTableT<kFastMaxGroups>*>(smem + C::SCHED_OFF);
@@ -121,13 +129,28 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
 #pragma unroll
   for (int k = 0; k < 8; ++k) vo[k] = Op::lane_voff(lane, wave % Op::NPAT, ld) + (wave + 4 * k) * Op::RPI * ld;
   static_assert(Op::NPAT == 2, "the swizzle pattern of copy wave + 4 k is that of copy wave");
+  // NN: B's copies have offsets of their own (two token rows of 512 bytes per copy, row pitch 2 N)
+  const int ld_b = (B_KMAJOR ? p.K : p.N) * 2;
+  int vo_b[B_KMAJOR ? 1 : 8];
+  if (!B_KMAJOR) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) vo_b[B_KMAJOR ? 0 : k] = OpB::lane_voff(lane, (wave + 4 * k) % OpB::NPAT, ld_b) + (wave + 4 * k) * OpB::RPI * ld_b;
+  }
 
   // LDS addresses of the fragment reads relative to a slab buffer (see gemm_fast.hip for the layout)
-  uint32_t a_rd[2], b_rd[2];
+  uint32_t a_rd[2], b_rd[B_KMAJOR ? 2 : 8];
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) {
-    a_rd[ks] = smem_addr + (wm0 + l16) * 128 + (((4 * ks + lg) ^ ((l16 / 2) % 8)) << 4);
-    b_rd[ks] = smem_addr + C::A_BYTES + (wn0 + l16) * 128 + (((4 * ks + lg) ^ ((l16 / 2) % 8)) << 4);
+  for (int ks = 0; ks < 2; ++ks) a_rd[ks] = smem_addr + (wm0 + l16) * 128 + (((4 * ks + lg) ^ ((l16 / 2) % 8)) << 4);
+  if (B_KMAJOR) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) b_rd[ks] = smem_addr + C::A_BYTES + (wn0 + l16) * 128 + (((4 * ks + lg) ^ ((l16 / 2) % 8)) << 4);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {  // per column block: token row 8 lg + e, 16-byte chunk of the lane's columns, swizzled
+      const int e = l16 >> 2, c = l16 & 3;
+      const int chunk = ((wn0 + 16 * j) / 8 + (c >> 1)) ^ (e * 4) ^ ((lg & 1) * 2);
+      b_rd[B_KMAJOR ? 0 : j] = smem_addr + C::A_BYTES + (lg * 8 + e) * (C::BN * 2) + chunk * 16 + (c & 1) * 8;
+    }
   }
 
   // ---- the copy stream --------------------------------------------------------------------------------------------
@@ -141,7 +164,10 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
     Win w;
     const int n_left = p.N - t.n0;
     w.rs = make_rsrc32((uint64_t)p.A + (uint64_t)(t.row0 * ld), live ? t.rows * ld : 0);  // only the tile's valid rows
-    w.rd = make_rsrc32((uint64_t)p.B + (uint64_t)(((int64_t)t.g * p.N + t.n0) * ld), live ? (n_left < C::BN ? n_left : C::BN) * ld : 0);
+    if (B_KMAJOR) w.rd = make_rsrc32((uint64_t)p.B + (uint64_t)(((int64_t)t.g * p.N + t.n0) * ld), live ? (n_left < C::BN ? n_left : C::BN) * ld : 0);
+    // NN: the tile's 256 columns of the group's K rows; N is a multiple of 256 (w4_supported), so every 512-byte row
+    // segment lies inside its row, and the scalar offset of a slab (which the range check leaves out) stays below K rows
+    else w.rd = make_rsrc32((uint64_t)p.B + (uint64_t)(((int64_t)t.g * p.K * p.N + t.n0) * 2), live ? p.K * ld_b : 0);
     return w;
   };
   const TileWalk walk64 = sched_walk(num_tiles, p.tile_split != 0);
@@ -198,14 +224,14 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   };
   auto copy_d = [&](auto Kc, const i32x4_t& rb, int koff, bool spaced) __attribute__((always_inline))  {
     constexpr int k = decltype(Kc)::value;
-    const int v = vo[k];
+    const int v = B_KMAJOR ? vo[k] : vo_b[B_KMAJOR ? 0 : k];
     if (spaced) asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(v), "s"(rb), "s"(koff) : "memory");
     else asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(v), "s"(rb), "s"(koff) : "memory");
   };
   // a slab's A copy k straight to LDS (prologue only)
-  auto copy_direct = [&](auto Kc, const i32x4_t& ra, int koff, uint32_t buf_addr) __attribute__((always_inline))  {
+  auto copy_direct = [&](auto Kc, auto ISBc, const i32x4_t& ra, int koff, uint32_t buf_addr) __attribute__((always_inline))  {
     constexpr int k = decltype(Kc)::value;
-    const int v = vo[k];
+    const int v = (B_KMAJOR || !decltype(ISBc)::value) ? vo[k] : vo_b[B_KMAJOR ? 0 : k];
     asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %3, %4 offen lds"
                  : : "s"(buf_addr), "n"(4 * k * 1024), "v"(v), "s"(ra), "s"(koff) : "memory", "m0", "scc");
   };
@@ -223,8 +249,12 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   // (the next step needs all of them at once), then A fragments in the order of use
   auto read_frag = [&](auto KSc, auto Qc, i32x4_t (&sa)[8], i32x4_t (&sb)[8], uint32_t buf_off) {
     constexpr int KS = decltype(KSc)::value, Q = decltype(Qc)::value;
-    if (Q < 8) lds_read_b128<Q * 2048>(sb[Q], b_rd[KS] + buf_off);
-    else lds_read_b128<(Q - 8) * 2048>(sa[Q - 8], a_rd[KS] + buf_off);
+    if (Q < 8) {
+      if (B_KMAJOR) lds_read_b128<Q * 2048>(sb[Q], b_rd[B_KMAJOR ? KS : 0] + buf_off);
+      else lds_read_tr<KS * 32 * (C::BN * 2), KS * 32 * (C::BN * 2) + 4 * (C::BN * 2)>(sb[Q], b_rd[B_KMAJOR ? 0 : (Q < 8 ? Q : 0)] + buf_off);
+    } else {
+      lds_read_b128<(Q - 8) * 2048>(sa[Q - 8], a_rd[KS] + buf_off);
+    }
   };
   // ---- deferred epilogue ---------------------------------------------------------------------------------------------
   // A tile's results are stored during the first K step of the workgroup's next tile: with one wave per SIMD nothing
@@ -315,9 +345,11 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
 #pragma unroll
     for (int q = 0; q < 3; ++q) rs_c[q] = wrap ? nxt.rs[q] : rs_c[q];
   };
+  const int d_step = B_KMAJOR ? 128 : __builtin_amdgcn_readfirstlane(64 * ld_b);         // B's slab offset per slab ...
+  const int d_bytes = B_KMAJOR ? k_bytes : __builtin_amdgcn_readfirstlane(p.K * ld_b);   // ... and where it reaches the next tile
   auto advance_d = [&]() __attribute__((always_inline))  {
-    const bool wrap = koff_d + 128 == k_bytes;
-    koff_d = wrap ? 0 : koff_d + 128;
+    const bool wrap = koff_d + d_step == d_bytes;
+    koff_d = wrap ? 0 : koff_d + d_step;
 #pragma unroll
     for (int q = 0; q < 3; ++q) rd_c[q] = wrap ? nxt.rd[q] : rd_c[q];
   };
@@ -397,8 +429,8 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
     rd_c = w0.rd;
   }
 #define TGG_W4_EACH(f) f(0) f(1) f(2) f(3) f(4) f(5) f(6) f(7)
-#define TGG_W4_P0(c) copy_direct(std::integral_constant<int, c>(), rs_c, 0, wave_buf + S_OFF); \
-                     copy_direct(std::integral_constant<int, c>(), rd_c, 0, wave_buf + D_OFF);
+#define TGG_W4_P0(c) copy_direct(std::integral_constant<int, c>(), No(), rs_c, 0, wave_buf + S_OFF); \
+                     copy_direct(std::integral_constant<int, c>(), Yes(), rd_c, 0, wave_buf + D_OFF);
   TGG_W4_EACH(TGG_W4_P0)
 #undef TGG_W4_P0
   wait_vmcnt<0>();
@@ -406,14 +438,14 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
 #define TGG_W4_P1(c) load_s(std::integral_constant<int, c>(), I1(), rs_c, 128);
   TGG_W4_EACH(TGG_W4_P1)
 #undef TGG_W4_P1
-#define TGG_W4_P2(c) copy_direct(std::integral_constant<int, c>(), rd_c, 128, wave_buf + C::STAGE_BYTES + D_OFF);
+#define TGG_W4_P2(c) copy_direct(std::integral_constant<int, c>(), Yes(), rd_c, d_step, wave_buf + C::STAGE_BYTES + D_OFF);
   TGG_W4_EACH(TGG_W4_P2)
 #undef TGG_W4_P2
 #define TGG_W4_P3(c) load_s(std::integral_constant<int, c>(), I0(), rs_c, 256);
   TGG_W4_EACH(TGG_W4_P3)
 #undef TGG_W4_P3
   koff_s = 3 * 128;  // at least four slabs per tile (w4_supported): both cursors are still in the first tile
-  koff_d = 2 * 128;
+  koff_d = 2 * d_step;
   kstep(I1(), I0(), No(), I0(), 0u, No(), 0u, I0(), 0u);  // reads K step 0 of buffer 0 into set 0, multiplies nothing, waits for everything
   const int kt_all = p.K / BK4;
 
@@ -484,7 +516,9 @@ int launch_w4(const GemmParams& p, hipStream_t s) {
 // kernels, which choose narrower tiles on the device.
 bool w4_supported(const GemmParams& p, int dt, int layout, bool any_size) {
   if (dt != DT_BF16 && dt != DT_F16) return false;
-  if (layout != W4_NT) return false;
+  if (layout != W4_NT && layout != W4_NN) return false;
+  // NN: every 512-byte row segment of a tile must lie inside its row of B, and a group's B within 2 GiB
+  if (layout == W4_NN && ((p.N & 255) != 0 || (int64_t)p.K * p.N * 2 >= (1ll << 31))) return false;
   if (p.mode != MODE_MG && p.mode != MODE_MG_PAD && p.mode != MODE_MASKED) return false;
   // masked launches are decided on the device, by a predicate that needs one thread of this kernel per group
   if (p.mode == MODE_MASKED && p.G > W4Cfg::THREADS) return false;
@@ -503,8 +537,12 @@ bool w4_supported(const GemmParams& p, int dt, int layout, bool any_size) {
 
 int launch_w4_16bit(const GemmParams& p, int dt, int layout, hipStream_t s) {
   const bool sit_out = p.mode == MODE_MASKED;
-  if (dt == DT_BF16) return sit_out ? launch_w4<DT_BF16, W4_NT, true>(p, s) : launch_w4<DT_BF16, W4_NT, false>(p, s);
-  return sit_out ? launch_w4<DT_F16, W4_NT, true>(p, s) : launch_w4<DT_F16, W4_NT, false>(p, s);
+  if (layout == W4_NT) {
+    if (dt == DT_BF16) return sit_out ? launch_w4<DT_BF16, W4_NT, true>(p, s) : launch_w4<DT_BF16, W4_NT, false>(p, s);
+    return sit_out ? launch_w4<DT_F16, W4_NT, true>(p, s) : launch_w4<DT_F16, W4_NT, false>(p, s);
+  }
+  if (dt == DT_BF16) return sit_out ? launch_w4<DT_BF16, W4_NN, true>(p, s) : launch_w4<DT_BF16, W4_NN, false>(p, s);
+  return sit_out ? launch_w4<DT_F16, W4_NN, true>(p, s) : launch_w4<DT_F16, W4_NN, false>(p, s);
 }
 
 }  // namespace tgg
