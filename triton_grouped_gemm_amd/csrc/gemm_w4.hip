@@ -271,15 +271,16 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   bool pending = false;
   char* const stage = smem + C::EPI_OFF + wave * C::EPI_WAVE_BYTES;
   // per-lane staging addresses and output offset, recomputed where a first K step or a flush begins
-  struct EpiLane { char* wr; const char* rd; int off; int ch8; };
+  struct EpiLane { char* wr; const char* rd; int off[2]; };  // off[h]: output offset of the lane's 16 bytes in column half h of strip 0, out of range where those columns lie beyond N
   auto epi_lane = [&]() __attribute__((always_inline))  {
     int el = lane;
     asm volatile("" : "+v"(el));
     EpiLane e;
     e.wr = stage + (el & 15) * C::EPI_PITCH + (el >> 4) * 8;
     e.rd = stage + (el >> 3) * C::EPI_PITCH + (el & 7) * 16;
-    e.off = ((el >> 3) * p.N + (el & 7) * 8) * 2;
-    e.ch8 = (el & 7) * 8;
+    const int off = ((el >> 3) * p.N + (el & 7) * 8) * 2, ch8 = (el & 7) * 8;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) e.off[h] = (64 * h + ch8 < pend_cols) ? off + 128 * h : kNoFetch;
     return e;
   };
   // block (i, j) -> staging piece j / 4; not before this point in the instruction stream
@@ -293,14 +294,15 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
     for (int it = 0; it < 2; ++it) v[it] = *(const i32x4_t*)(e.rd + h * C::EPI_PIECE + it * 8 * C::EPI_PITCH);
     asm volatile("" ::: "memory");
   };
-  auto epi_store = [&](const EpiLane& e, int i, int h, int it, const i32x4_t& v) __attribute__((always_inline))  {
-    const int off = (64 * h + e.ch8 < pend_cols) ? e.off + ((16 * i + 8 * it) * p.N + 64 * h) * 2 : kNoFetch;
-    i32x4_t rs;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) rs[q] = __builtin_amdgcn_readfirstlane(pend_rs[q]);
-    // the wait states in front cover a descriptor written by a vector instruction just before (the compiler does not
-    // space what sits inside this statement), those behind it keep the data registers intact until the store has them
-    asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, 0 offen nt\n\ts_nop 1" : : "v"(v), "v"(off), "s"(rs) : "memory");
+  auto epi_store = [&](const EpiLane& e, int i, int h, int it, const i32x4_t& v, bool between_multiplies) __attribute__((always_inline))  {
+    // (an out-of-range marker stays out of range with the rows' offset added: both are far below 2^31)
+    const int off = e.off[h] + (16 * i + 8 * it) * p.N * 2;
+    // Two wait states must pass before a 16-byte store's data registers may be overwritten, and the compiler, which
+    // considers them free after this statement, reuses them at once: between multiplies the multiply that follows is
+    // one wait state, the flush has none.  No wait states in front: the descriptor sits in scalar registers since the
+    // end of the tile.  Both hazards are checked on the kept assembly (tests/test_isa_hazards.py).
+    if (between_multiplies) asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen nt\n\ts_nop 0" : : "v"(v), "v"(off), "s"(pend_rs) : "memory");
+    else asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen nt\n\ts_nop 1" : : "v"(v), "v"(off), "s"(pend_rs) : "memory");
   };
   // everything that is pending, without multiplies to hide it under
   auto epi_flush = [&]() __attribute__((always_inline))  {
@@ -317,8 +319,8 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
         for (int h = 0; h < 2; ++h) {
           i32x4_t v[2];
           epi_read(e, h, v);
-          epi_store(e, i, h, 0, v[0]);
-          epi_store(e, i, h, 1, v[1]);
+          epi_store(e, i, h, 0, v[0], false);
+          epi_store(e, i, h, 1, v[1], false);
         }
       }
     }
@@ -369,7 +371,7 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
     constexpr int CUR = decltype(CURc)::value, NKS = decltype(NKSc)::value, ROLE = decltype(ROLEc)::value;
     constexpr bool MUL = decltype(MULc)::value, EPI = decltype(EPIc)::value;
     static_assert(!EPI || MUL, "the deferred epilogue rides on a multiplying K step");
-    EpiLane e = {nullptr, nullptr, 0, 0};
+    EpiLane e = {nullptr, nullptr, {0, 0}};
     i32x4_t v0[2], v1[2];
     if (EPI) {
       e = epi_lane();
@@ -385,10 +387,10 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
           if (jj == 0) epi_read(e, 0, v0);            // strip i, staged during the previous row block
           if (jj == 1) epi_read(e, 1, v1);
           if (i < 7) epi_cvt(e, i + 1, jj);           // its piece's read-back has been issued (jj = 0: piece 0, jj = 4: piece 1)
-          if (jj == 3) epi_store(e, i, 0, 0, v0[0]);
-          if (jj == 4) epi_store(e, i, 0, 1, v0[1]);
-          if (jj == 5) epi_store(e, i, 1, 0, v1[0]);
-          if (jj == 6) epi_store(e, i, 1, 1, v1[1]);
+          if (jj == 3) epi_store(e, i, 0, 0, v0[0], true);
+          if (jj == 4) epi_store(e, i, 0, 1, v0[1], true);
+          if (jj == 5) epi_store(e, i, 1, 0, v1[0], true);
+          if (jj == 6) epi_store(e, i, 1, 1, v1[1], true);
           mfma_new<DT>(acc[i][j], fb[CUR][j], fa[CUR][i]);
         } else if (MUL) {
           mfma_acc<DT>(acc[i][j], fb[CUR][j], fa[CUR][i]);
