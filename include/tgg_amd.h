@@ -238,7 +238,7 @@ int tgg_debug_queue_order(int grid, int draws, int32_t* out);
  *                        the persistent workgroups, at 0.7 of a 256-row tile's cost each, are no more than those of
  *                        the 256x256 tiles (groups of up to about 200 rows on average); 256x256 otherwise; 1 = always 256x128; 2 = always 256x256; 4 = always the weight-streaming
  *                        configuration (16-bit NT / NN, FP8 M-grouped)
- *   "four_wave"     int  16-bit M-grouped / masked NT with K a multiple of 128 (at least 256): 1 (default) = the four-wave
+ *   "four_wave"     int  16-bit M-grouped / masked NT (or NN with N a multiple of 256), K a multiple of 128 (at least 256): 1 (default) = the four-wave
  *                        kernel (128x128 per wave) on large launches (more than four rounds of 256x128 tiles; M-grouped:
  *                        at least 512 rows per group on average; masked: both kernels are enqueued and decide on the
  *                        device from masked_m which of them runs), 0 = eight-wave kernels only, 2 = the four-wave

@@ -1,4 +1,5 @@
-// Four-wave bf16/fp16 grouped GEMM kernel for gfx950: the large-problem path of the M-grouped NT entry points.
+// Four-wave bf16/fp16 grouped GEMM kernel for gfx950: the large-problem path of the M-grouped and masked entry points
+// (B as [G, N, K], or as [G, K, N] with N a multiple of 256).
 //
 // One workgroup per CU, four waves, one per SIMD; tile 256x256, K slab 64; every wave owns a 128x128 block of
 // 16x16x32 MFMA tiles with its 256 accumulator registers in AGPRs.  Against the eight-wave kernel (gemm_fast.hip,
