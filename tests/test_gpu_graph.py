@@ -112,6 +112,45 @@ def test_group_sizes_may_change_between_replays(dev):
         assert bool((out16[rows:] == 7.0).all()) and bool((out8[placed:] == 7.0).all()), f"replay {it}: rows past the groups"
 
 
+def test_masked_counts_may_change_which_kernel_runs_between_replays(dev):
+    """A masked launch of this size enqueues the four-wave kernel and the eight-wave kernel, and the counts decide on
+    the device which of them does the work.  One captured graph holds both launches; between replays masked_m is
+    rewritten so that the choice flips (counts near m_max: 256-row tiles pay; a few dozen rows per group: they do not)."""
+    G, m_max, N, K = 72, 512, 1032, 256
+    lhs = torch.randint(-1, 2, (G * m_max, K), generator=torch.Generator().manual_seed(41)).to(torch.bfloat16).to(dev)
+    rhs = torch.randint(-1, 2, (G, N, K), generator=torch.Generator().manual_seed(42)).to(torch.bfloat16).to(dev)
+    ref = torch.bmm(lhs.float().view(G, m_max, K), rhs.float().transpose(1, 2)).to(torch.bfloat16)  # exact: integers
+    masked = torch.zeros(G, dtype=torch.int32, device=dev)
+    out = torch.empty((G * m_max, N), dtype=torch.bfloat16, device=dev)
+
+    def step():
+        _native.call("tgg_m_grouped_gemm_masked", lhs.data_ptr(), rhs.data_ptr(), out.data_ptr(), masked.data_ptr(), 0, G,
+                     m_max, G * m_max, N, K, 1, _native.DTYPE_CODE[torch.bfloat16], -1, _native.stream_of(lhs))
+
+    counts = [
+        [512 - (37 * g) % 200 for g in range(G)],
+        [(53 * g) % 100 for g in range(G)],
+        [(131 * g) % 513 for g in range(G)],
+        [0] * G,
+    ]
+    masked.copy_(torch.tensor(counts[0], dtype=torch.int32))
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for it, c in enumerate(counts * 2):
+        masked.copy_(torch.tensor(c, dtype=torch.int32))
+        out.fill_(-5.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.view(G, m_max, N)
+        for g, mm in enumerate(c):
+            assert torch.equal(got[g, :mm], ref[g, :mm]), f"replay {it} group {g}"
+            assert bool((got[g, mm:] == -5.0).all()), f"replay {it} group {g}: rows beyond masked_m were written"
+
+
 def test_deep_gemm_shaped_wrappers_can_be_captured(dev):
     """m_grouped_bf16_nt_contiguous / m_grouped_fp8_nt_contiguous check M against the padded sizes on the host, as
     the reference does; under capture that read is left out, so the wrappers themselves can sit in a graph (with
