@@ -239,10 +239,10 @@ int tgg_debug_queue_order(int grid, int draws, int32_t* out);
  *                        the 256x256 tiles (groups of up to about 200 rows on average); 256x256 otherwise; 1 = always 256x128; 2 = always 256x256; 4 = always the weight-streaming
  *                        configuration (16-bit NT / NN, FP8 M-grouped)
  *   "four_wave"     int  16-bit M-grouped / masked NT (or NN with N a multiple of 256), K a multiple of 128 (at least 256): 1 (default) = the four-wave
- *                        kernel (128x128 per wave) on large launches (more than four rounds of 256x128 tiles; M-grouped:
- *                        at least 512 rows per group on average; masked: both kernels are enqueued and decide on the
- *                        device from masked_m which of them runs), 0 = eight-wave kernels only, 2 = the four-wave
- *                        kernel on every launch it can take, whatever the sizes
+ *                        kernel (128x128 per wave) on large launches (more than four rounds of 256x128 tiles; masked
+ *                        launches and M-grouped ones with fewer than 512 rows per group on average enqueue both
+ *                        kernels, which decide on the device from the sizes which of them runs), 0 = eight-wave
+ *                        kernels only, 2 = the four-wave kernel on every launch it can take, whatever the sizes
  *   "tile_split"    0/1  M-grouped tuned kernels: per-XCD contiguous tile ranges (default 1) or interleaved sweeps
  *   "n_chunk"       int  column tiles per chunk of the tile order (0 = automatic, at most eight)
  *   "store_nt"      0/1  write the output with non-temporal stores (default 1)

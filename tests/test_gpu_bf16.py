@@ -338,6 +338,28 @@ def test_masked_decode_sized_counts(dev):
         assert bool((out[g, mm:] == -5.0).all()), f"group {g}: rows beyond masked_m were written"
 
 
+@pytest.mark.parametrize("trans_b", [True, False])
+def test_m_grouped_launch_that_both_kernels_look_at(dev, trans_b):
+    """An M-grouped launch with many tiles but fewer than 512 rows per group on average: like a masked one it enqueues
+    the four-wave and the eight-wave kernel and the sizes decide on the device which runs (here: groups of up to 700
+    rows, 256-row tiles pay).  Exact on integer inputs; the same bits as either kernel forced."""
+    G, N, K = 96, 1024, 256
+    sizes = [(131 * g) % 700 for g in range(G)]
+    M = sum(sizes)
+    assert M < 512 * G
+    a = _ints((M, K), 51)
+    b = _ints((G, N, K) if trans_b else (G, K, N), 52)
+    ref = gemm_ref.gmm_fp32(a, b, sizes, trans_b).to(torch.bfloat16)
+    s_dev, a_dev, b_dev = torch.tensor(sizes, dtype=torch.int32, device=dev), a.to(dev), b.to(dev)
+    for four_wave in (1, 2, 0):
+        _native.set_option("four_wave", four_wave)
+        try:
+            out = m_grouped_gemm(a_dev, b_dev, s_dev, trans_b)
+        finally:
+            _native.set_option("four_wave", 1)
+        assert torch.equal(out.cpu(), ref), f"four_wave={four_wave}"
+
+
 @pytest.mark.parametrize("counts", ["large", "small", "mixed"])
 def test_masked_launch_that_both_kernels_look_at(dev, counts):
     """A masked launch large enough for the four-wave kernel (K a multiple of 128, many tiles): it and the eight-wave

@@ -58,6 +58,7 @@ int launch_cvt_fp8(const float*, void*, int64_t, int, hipStream_t);
 bool fast_supported(const GemmParams& p, int dt, int layout);
 int launch_fast_16bit(const GemmParams& p, int dt, int layout, hipStream_t s);
 bool w4_supported(const GemmParams& p, int dt, int layout, bool any_size);
+bool w4_decided_on_device(const GemmParams& p);
 int launch_w4_16bit(const GemmParams& p, int dt, int layout, hipStream_t s);
 bool fast_quant_supported(const GemmParams& p, int dt, int layout);
 int launch_fast_16bit_quant(const GemmParams& p, int dt, int layout, hipStream_t s);
@@ -177,8 +178,8 @@ static GemmParams params_fp8_block(const void* Aq, const float* sa, const void* 
 static int dispatch_16bit(const GemmParams& p, int dt, int layout, hipStream_t s) {
   const int force_generic = g_force_generic.load(), four_wave = g_four_wave.load();
   if (!force_generic && four_wave && w4_supported(p, dt, layout, four_wave == 2)) {
-    if (p.mode != MODE_MASKED || four_wave == 2) return launch_w4_16bit(p, dt, layout, s);
-    // masked: whether 256-row tiles pay depends on the counts; both kernels look at them and exactly one runs
+    if (!w4_decided_on_device(p) || four_wave == 2) return launch_w4_16bit(p, dt, layout, s);
+    // whether 256-row tiles pay depends on the sizes; both kernels look at them and exactly one runs
     GemmParams q = p;
     q.wide_gate = 1;
     if (int e = launch_w4_16bit(q, dt, layout, s)) return e;

@@ -104,8 +104,9 @@ struct GemmParams {
   // counts, so both kernels are launched and each looks at the counts first: 1 = run only if all counts are
   // multiples of 16 (tuned), 2 = run only if one is not (shape-agnostic), 0 = always run.
   int kg_gate;
-  // Masked 16-bit launches that the four-wave kernel could take: it pays only where the eight-wave kernels would
-  // choose their 256x256 tiles, which depends on the counts, and only the device knows them.  Both kernels are
+  // 16-bit launches that the four-wave kernel could take but whose groups may be small (masked; M-grouped with fewer
+  // than 512 rows per group on average): it pays only where the eight-wave kernels would choose their 256x256 tiles,
+  // which depends on the sizes, and only the device knows them.  Both kernels are
   // launched and each evaluates the same predicate on its group table first (sched_wide_tiles_chosen):
   // 1 = run only if it holds (four-wave), 2 = run only if it does not (eight-wave), 0 = always run.
   int wide_gate;

@@ -514,6 +514,13 @@ int launch_w4(const GemmParams& p, hipStream_t s) {
 
 }  // namespace
 
+// Whether 256-row tiles pay depends on the group sizes, which only the device knows.  With 512 rows and more per group on
+// average they do; a masked launch (counts anywhere up to its row stride) or an M-grouped one with smaller groups is
+// enqueued together with the eight-wave kernel, and the two decide from the sizes which of them runs.
+bool w4_decided_on_device(const GemmParams& p) {
+  return p.mode == MODE_MASKED || p.m_total < 512 * (int64_t)p.G;
+}
+
 // The four-wave kernel takes M-grouped launches (rows contiguous or padded) whose tile count is large whatever the
 // group sizes turn out to be: at least ceil(m_total / 256) row tiles.  Smaller launches stay with the eight-wave
 // kernels, which choose narrower tiles on the device.
@@ -523,8 +530,9 @@ bool w4_supported(const GemmParams& p, int dt, int layout, bool any_size) {
   // NN: every 512-byte row segment of a tile must lie inside its row of B, and a group's B within 2 GiB
   if (layout == W4_NN && ((p.N & 255) != 0 || (int64_t)p.K * p.N * 2 >= (1ll << 31))) return false;
   if (p.mode != MODE_MG && p.mode != MODE_MG_PAD && p.mode != MODE_MASKED) return false;
-  // masked launches are decided on the device, by a predicate that needs one thread of this kernel per group
-  if (p.mode == MODE_MASKED && p.G > W4Cfg::THREADS) return false;
+  // launches whose groups may be small are decided on the device (w4_decided_on_device), by a predicate that needs
+  // one thread of this kernel per group
+  if (w4_decided_on_device(p) && p.G > W4Cfg::THREADS) return false;
   if (p.q_fmt != 0 || p.G > kFastMaxGroups) return false;
   if ((p.N & 7) != 0 || p.K < 8 || (p.K & 7) != 0) return false;
   if ((int64_t)p.K * 2 * 256 >= (1ll << 30)) return false;
@@ -534,8 +542,7 @@ bool w4_supported(const GemmParams& p, int dt, int layout, bool any_size) {
   if (p.grid_limit > 0 && p.grid_limit < grid) grid = p.grid_limit;
   const int64_t row_tiles = (p.m_total + 255) / 256;
   const int64_t narrow_tiles = row_tiles * ((p.N + 127) / 128);
-  // groups of 512 rows and more on average: where the eight-wave kernels would choose 256-row tiles as well
-  return narrow_tiles > 4 * (int64_t)grid && (p.mode == MODE_MASKED || p.m_total >= 512 * (int64_t)p.G);
+  return narrow_tiles > 4 * (int64_t)grid;
 }
 
 int launch_w4_16bit(const GemmParams& p, int dt, int layout, hipStream_t s) {
