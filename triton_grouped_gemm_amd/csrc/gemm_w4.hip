@@ -20,6 +20,9 @@
 //   wait for the fragment reads and for this wave's B copies of slab r+1, workgroup barrier
 //   K step 1   64 multiplies on set 1; meanwhile the fragments of slab r+1 / K step 0 are read into set 0 and
 //              this wave's B copies of slab r+2 go straight to LDS, into the buffer of slab r
+// Within a K step the sixteen fragment reads follow the first sixteen multiplies, one each; the LDS writes with their
+// reloads, or the copies, follow from the seventeenth multiply on, one every fourth or fifth multiply (fragment
+// reads and 16-byte LDS writes slow each other down when they alternate).
 // A is the operand that streams from memory (B panels are shared through L2), so it is requested two slabs
 // earlier than an LDS buffer is free for it: worth 3 % over copying it straight to LDS a slab ahead, although
 // the LDS writes cost more than that copy would.  The slabs of all of a workgroup's tiles form one stream; each
@@ -29,9 +32,9 @@
 // tile's first K step (see "deferred epilogue" below), whose multiplies start from a zero addend instead of the
 // accumulators.  That K step is the one place where a gap holds a dozen instructions (8 % of a launch).
 //
-// Headline shape (G = 128, M = 655360, N = 1536, K = 2048), same box: 3.18 ms against 3.30 ms for the eight-wave
-// kernel; K = 768 shape 1.91 against 1.97 ms; masked decode (G = 128, up to 512 rows per group, N = 4096, K = 1536)
-// 0.53 against 0.56 ms.  Large M-grouped launches with K a multiple of 128 take this kernel (w4_supported); masked
+// Headline shape (G = 128, M = 655360, N = 1536, K = 2048), same box: 3.11 ms against 3.30 ms for the eight-wave
+// kernel; K = 768 shape 1.88 against 1.97 ms; masked decode (G = 128, up to 512 rows per group, N = 4096, K = 1536)
+// 0.52 against 0.56 ms.  Large M-grouped launches with K a multiple of 128 take this kernel (w4_supported); masked
 // launches of that size enqueue it together with the eight-wave kernel and the counts decide on the device which of
 // the two runs (GemmParams::wide_gate); everything else goes to the eight-wave kernels.
 //
@@ -358,8 +361,11 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   };
 
   // One K step: 64 multiplies on fragment set CUR (when MUL); the 16 fragments of K step NKS of the slab at nb_off go
-  // to the other set, one read every third multiply.  At most two other instructions sit between two multiplies: a
-  // wave issues in order, and what exceeds the sixteen cycles of a multiply leaves the matrix pipe idle.
+  // to the other set, one read after each of the first sixteen multiplies; the LDS writes and the loads and copies follow
+  // behind them (reads and staged writes apart in time: 2.5 % over interleaving them through the whole K step; the
+  // loads must not slip much later, a quarter of a slab less lead costs 6 %).  At most two other instructions sit
+  // between two multiplies: a wave issues in order, and what exceeds the sixteen cycles of a multiply leaves the matrix
+  // pipe idle.
   // ROLE 0: prologue (reads only, waits for everything).
   // ROLE 1: a slab's first K step.  The A chunks of the next slab go from register set SET to LDS (wr_addr) and the
   //         chunks of the slab three ahead are requested into the same set; ends with the wait for the B copies of
@@ -397,23 +403,23 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
           mfma_acc<DT>(acc[i][j], fb[CUR][j], fa[CUR][i]);
         }
         const int n = i * 8 + jj;
-#define TGG_W4_RD(q) if (n + 1 == 3 * (q + 1)) read_frag(std::integral_constant<int, NKS>(), std::integral_constant<int, q>(), fa[CUR ^ 1], fb[CUR ^ 1], nb_off);
+#define TGG_W4_RD(q) if (n == q) read_frag(std::integral_constant<int, NKS>(), std::integral_constant<int, q>(), fa[CUR ^ 1], fb[CUR ^ 1], nb_off);
         TGG_W4_RD(0) TGG_W4_RD(1) TGG_W4_RD(2) TGG_W4_RD(3) TGG_W4_RD(4) TGG_W4_RD(5) TGG_W4_RD(6) TGG_W4_RD(7)
         TGG_W4_RD(8) TGG_W4_RD(9) TGG_W4_RD(10) TGG_W4_RD(11) TGG_W4_RD(12) TGG_W4_RD(13) TGG_W4_RD(14) TGG_W4_RD(15)
 #undef TGG_W4_RD
         if (ROLE == 1) {
-#define TGG_W4_ST(c) if (n == 6 * c + 1) write_s(std::integral_constant<int, c>(), SETc, wr_addr); \
-                     if (n == 6 * c + 4) { load_s(std::integral_constant<int, c>(), SETc, rs_c, koff_s); if (!MUL) __builtin_amdgcn_s_sleep(1); }
+#define TGG_W4_ST(c) if (n == 16 + 4 * c) write_s(std::integral_constant<int, c>(), SETc, wr_addr); \
+                     if (n == 18 + 4 * c) { load_s(std::integral_constant<int, c>(), SETc, rs_c, koff_s); if (!MUL) __builtin_amdgcn_s_sleep(1); }
           TGG_W4_ST(0) TGG_W4_ST(1) TGG_W4_ST(2) TGG_W4_ST(3) TGG_W4_ST(4) TGG_W4_ST(5) TGG_W4_ST(6) TGG_W4_ST(7)
 #undef TGG_W4_ST
           if (n == 52) advance_s();
         }
         if (ROLE == 2) {
-#define TGG_W4_CP(c) if (n == 6 * c + 3) copy_d_m0(std::integral_constant<int, c>(), cp_addr); \
-                     if (n == 6 * c + 4) { copy_d(std::integral_constant<int, c>(), rd_c, koff_d, MUL); if (!MUL) __builtin_amdgcn_s_sleep(1); }
+#define TGG_W4_CP(c) if (n == 16 + 5 * c) copy_d_m0(std::integral_constant<int, c>(), cp_addr); \
+                     if (n == 17 + 5 * c) { copy_d(std::integral_constant<int, c>(), rd_c, koff_d, MUL); if (!MUL) __builtin_amdgcn_s_sleep(1); }
           TGG_W4_CP(0) TGG_W4_CP(1) TGG_W4_CP(2) TGG_W4_CP(3) TGG_W4_CP(4) TGG_W4_CP(5) TGG_W4_CP(6) TGG_W4_CP(7)
 #undef TGG_W4_CP
-          if (n == 52) advance_d();
+          if (n == 56) advance_d();
         }
       }
     if (ROLE == 2) asm volatile("s_waitcnt lgkmcnt(0)" : TGG_TIE8(fa[CUR ^ 1]), TGG_TIE8(fb[CUR ^ 1]) : : "memory");
