@@ -28,13 +28,20 @@
 // the LDS writes cost more than that copy would.  The slabs of all of a workgroup's tiles form one stream; each
 // of the two cursors carries the buffer descriptor of its tile's window and an offset along K.
 //
-// The epilogue is deferred: a tile's results are converted, staged and stored between the multiplies of the next
-// tile's first K step (see "deferred epilogue" below), whose multiplies start from a zero addend instead of the
-// accumulators.  That K step is the one place where a gap holds a dozen instructions (8 % of a launch).
+// The epilogue rides on multiplies: the upper half of a wave's block is converted and stored between the multiplies
+// of the tile's last K step, the lower half between those of the next tile's first K step, whose multiplies start
+// from a zero addend instead of the accumulators (see "epilogue" below).  With B as [G, N, K] the results never pass
+// through LDS: the rows of a B slab sit in LDS in an order that makes each lane's results of the eight column blocks
+// eight neighbouring outputs of a row.  Measured on the headline shape: staging a tile's results in LDS costs 9 % of
+// a launch in LDS bandwidth however it is spread over those two K steps (fragment reads already take half of it);
+// exchanging halves between lane groups instead gives 16 rows x 64 bytes per store, whose lanes four by four lie in
+// different rows, and costs 6 % more than staging; the permuted slab rows give 4 rows x 256 bytes per store and
+// cost nothing.  What remains of the epilogue is the write traffic itself (6 % of a launch against stores that
+// write nothing).
 //
-// Headline shape (G = 128, M = 655360, N = 1536, K = 2048), same box: 3.11 ms against 3.30 ms for the eight-wave
-// kernel; K = 768 shape 1.88 against 1.97 ms; masked decode (G = 128, up to 512 rows per group, N = 4096, K = 1536)
-// 0.52 against 0.56 ms.  Large M-grouped launches with K a multiple of 128 take this kernel (w4_supported); masked
+// Headline shape (G = 128, M = 655360, N = 1536, K = 2048), same box: 3.03 ms against 3.30 ms for the eight-wave
+// kernel; K = 768 shape 1.77 against 1.97 ms; masked decode (G = 128, up to 512 rows per group, N = 4096, K = 1536)
+// 0.51 against 0.56 ms.  Large M-grouped launches with K a multiple of 128 take this kernel (w4_supported); masked
 // launches of that size enqueue it together with the eight-wave kernel and the counts decide on the device which of
 // the two runs (GemmParams::wide_gate); everything else goes to the eight-wave kernels.
 //
@@ -45,9 +52,9 @@
 //     in the instruction text and listed as clobbered, the compiler never holds a value in them
 //     (tests/test_isa_hazards.py scans the kept assembly for any other use);
 //   * the multiplies write AGPRs: compiled code (the epilogue's conversions) reads a block's accumulators no sooner
-//     than 48 multiplies after the multiply that wrote them, except where a flush follows a tile directly: there the
-//     last row block's accumulators pass through a statement of idle cycles first.  Accumulators are never the
-//     target of a load.
+//     than three multiplies after the multiply that wrote them (a multiply takes 16 cycles to issue and delivers
+//     within two more), except where a flush follows a tile directly: there the last row block's accumulators pass
+//     through a statement of idle cycles first.  Accumulators are never the target of a load.
 #include "fast_common.hpp"
 #include "launch.hpp"
 
@@ -135,10 +142,19 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   static_assert(Op::NPAT == 2, "the swizzle pattern of copy wave + 4 k is that of copy wave");
   // NN: B's copies have offsets of their own (two token rows of 512 bytes per copy, row pitch 2 N)
   const int ld_b = (B_KMAJOR ? p.K : p.N) * 2;
-  int vo_b[B_KMAJOR ? 1 : 8];
-  if (!B_KMAJOR) {
+  // NT: B's rows land in LDS permuted: LDS row 128 h + 16 j + c of the slab (column block j of a wave's half h, lane
+  // column c of the multiply) holds column 128 h + 8 c + j of the tile, so that a lane's results of the eight column
+  // blocks are eight neighbouring outputs of a row and leave as one 16-byte store without passing through LDS.
+  int vo_b[8];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) vo_b[B_KMAJOR ? 0 : k] = OpB::lane_voff(lane, (wave + 4 * k) % OpB::NPAT, ld_b) + (wave + 4 * k) * OpB::RPI * ld_b;
+  for (int k = 0; k < 8; ++k) {
+    if (B_KMAJOR) {
+      const int r_local = lane / Op::CPR;  // LDS row 8 (wave + 4 k) + r_local: h = k / 4, j = 2 (k % 4) + wave / 2, c = 8 (wave % 2) + r_local
+      const int col = 128 * (k >> 2) + 8 * (8 * (wave & 1) + r_local) + 2 * (k & 3) + (wave >> 1);
+      vo_b[k] = Op::lane_voff(lane, wave % Op::NPAT, ld) + (col - r_local) * ld;
+    } else {
+      vo_b[k] = OpB::lane_voff(lane, (wave + 4 * k) % OpB::NPAT, ld_b) + (wave + 4 * k) * OpB::RPI * ld_b;
+    }
   }
 
   // LDS addresses of the fragment reads relative to a slab buffer (see gemm_fast.hip for the layout)
@@ -228,14 +244,14 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   };
   auto copy_d = [&](auto Kc, const i32x4_t& rb, int koff, bool spaced) __attribute__((always_inline))  {
     constexpr int k = decltype(Kc)::value;
-    const int v = B_KMAJOR ? vo[k] : vo_b[B_KMAJOR ? 0 : k];
+    const int v = vo_b[k];
     if (spaced) asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(v), "s"(rb), "s"(koff) : "memory");
     else asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(v), "s"(rb), "s"(koff) : "memory");
   };
   // a slab's A copy k straight to LDS (prologue only)
   auto copy_direct = [&](auto Kc, auto ISBc, const i32x4_t& ra, int koff, uint32_t buf_addr) __attribute__((always_inline))  {
     constexpr int k = decltype(Kc)::value;
-    const int v = (B_KMAJOR || !decltype(ISBc)::value) ? vo[k] : vo_b[B_KMAJOR ? 0 : k];
+    const int v = decltype(ISBc)::value ? vo_b[k] : vo[k];
     asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %3, %4 offen lds"
                  : : "s"(buf_addr), "n"(4 * k * 1024), "v"(v), "s"(ra), "s"(koff) : "memory", "m0", "scc");
   };
@@ -260,15 +276,22 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
       lds_read_b128<(Q - 8) * 2048>(sa[Q - 8], a_rd[KS] + buf_off);
     }
   };
-  // ---- deferred epilogue ---------------------------------------------------------------------------------------------
-  // A tile's results are stored during the first K step of the workgroup's next tile: with one wave per SIMD nothing
-  // else would keep the matrix pipe busy while a wave converts and stores its 128x128 block.  A lane owns row l16 and
-  // columns 16 j + 4 lg + (0..3) of each 16-row block i.  Strip i (one 16-row block, 128 columns) goes through the
+  // ---- epilogue ------------------------------------------------------------------------------------------------------
+  // With one wave per SIMD nothing else would keep the matrix pipe busy while a wave converts and stores its 128x128
+  // block, so the work sits in the gaps between multiplies: strips 0-3 (a strip: one 16-row block, 128 columns) during
+  // the tile's last K step, each after its last multiply, strips 4-7 during the first K step of the workgroup's next
+  // tile, each before the multiply that starts it afresh (that K step multiplies with a zero addend); a wave without
+  // a next tile to multiply stores strips 4-7 in a flush.  Half a block's conversion per gap on average keeps the
+  // gaps within what a multiply hides.
+  // B as [G, N, K]: the multiply takes A's fragment as its first operand, so a lane holds rows 16 i + 4 lg + r
+  // (r = 0..3) of one column per block, and the permuted slab rows (vo_b) make that column 8 l16 + j for block j:
+  // the lane's eight blocks of a strip are 16 contiguous bytes of an output row, 16 lanes cover 256 bytes of it, and
+  // a store instruction writes 4 rows x 256 bytes.
+  // B as [G, K, N] (fragments come from transposing reads, which tie a lane's column to its number): B's fragment is
+  // the first operand, a lane owns row l16 and columns 16 j + 4 lg + (0..3) of block (i, j); a strip goes through the
   // wave's LDS staging as two pieces of 64 columns and leaves as 16-byte stores covering 128-byte row segments.
-  // During the multiplies of row block i the blocks of strip i+1 are converted and staged one per multiply (their
-  // accumulators are the next to be overwritten: the first K step multiplies with a zero addend) and strip i,
-  // staged a row block earlier, is read back and stored.  The stores go through a buffer descriptor over the wave's
-  // block that ends with its last valid row; lanes whose columns lie beyond N get an out-of-range offset: no branches.
+  // The stores go through a buffer descriptor over the wave's block that ends with its last valid row; lanes whose
+  // columns lie beyond N get an out-of-range offset: no branches.
   // Nothing pending = a descriptor of length zero.
   i32x4_t pend_rs = make_rsrc32(0, 0);
   int pend_cols = 0;
@@ -308,15 +331,49 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
     if (between_multiplies) asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen nt\n\ts_nop 0" : : "v"(v), "v"(off), "s"(pend_rs) : "memory");
     else asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen nt\n\ts_nop 1" : : "v"(v), "v"(off), "s"(pend_rs) : "memory");
   };
+  // NT: no staging.  A lane holds rows 16 i + 4 lg + r (r = 0..3) of column 8 l16 + j of the wave's block in
+  // accumulator block (i, j), component r: the eight blocks of a strip give eight neighbouring outputs of a row.
+  auto epi_lane_t = [&]() __attribute__((always_inline))  {
+    int el = lane;
+    asm volatile("" : "+v"(el));
+    const int col = (el & 15) * 8;
+    return col < pend_cols ? ((el >> 4) * 4 * p.N + col) * 2 : kNoFetch;
+  };
+  // outputs 4 h .. 4 h + 3 of the lane's eight in row r of strip i, converted; not before this point in the instruction stream
+  auto epi_half_t = [&](int i, int r, int h) __attribute__((always_inline))  {
+    asm volatile("" : "+a"(acc[i][4 * h]), "+a"(acc[i][4 * h + 1]), "+a"(acc[i][4 * h + 2]), "+a"(acc[i][4 * h + 3]));
+    uint2 x;
+    x.x = pack2<DT>(acc[i][4 * h][r], acc[i][4 * h + 1][r]);
+    x.y = pack2<DT>(acc[i][4 * h + 2][r], acc[i][4 * h + 3][r]);
+    asm volatile("" : "+v"(x.x), "+v"(x.y));
+    return x;
+  };
+  auto epi_store_t = [&](int lane_off, int i, int r, const uint2& x, const uint2& y, bool between_multiplies) __attribute__((always_inline))  {
+    i32x4_t v;
+    v[0] = (int)x.x; v[1] = (int)x.y; v[2] = (int)y.x; v[3] = (int)y.y;
+    const int off = lane_off + (16 * i + r) * p.N * 2;
+    if (between_multiplies) asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen nt\n\ts_nop 0" : : "v"(v), "v"(off), "s"(pend_rs) : "memory");
+    else asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen nt\n\ts_nop 1" : : "v"(v), "v"(off), "s"(pend_rs) : "memory");
+  };
   // everything that is pending, without multiplies to hide it under
   auto epi_flush = [&]() __attribute__((always_inline))  {
     if (pending) {
       // the last row block's multiplies may have just been issued: give them time before compiled code reads the registers
       asm volatile("s_nop 15\n\ts_nop 7" : "+a"(acc[7][0]), "+a"(acc[7][1]), "+a"(acc[7][2]), "+a"(acc[7][3]),
                    "+a"(acc[7][4]), "+a"(acc[7][5]), "+a"(acc[7][6]), "+a"(acc[7][7]));
+      if (B_KMAJOR) {
+        const int lane_off = epi_lane_t();
+#pragma unroll
+        for (int i = 4; i < 8; ++i)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const uint2 x = epi_half_t(i, r, 0), y = epi_half_t(i, r, 1);
+            epi_store_t(lane_off, i, r, x, y, false);
+          }
+      }
       const EpiLane e = epi_lane();
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = B_KMAJOR ? 8 : 4; i < 8; ++i) {  // the first four strips left during the tile's last K step
 #pragma unroll
         for (int j = 0; j < 8; ++j) epi_cvt(e, i, j);
 #pragma unroll
@@ -369,38 +426,66 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   // ROLE 0: prologue (reads only, waits for everything).
   // ROLE 1: a slab's first K step.  The A chunks of the next slab go from register set SET to LDS (wr_addr) and the
   //         chunks of the slab three ahead are requested into the same set; ends with the wait for the B copies of
-  //         the next slab (eight younger loads, and 32 stores in a tile's first K step, may stay in flight; loads
+  //         the next slab (eight younger loads, and the 16 stores of a tile's first K step, may stay in flight; loads
   //         and stores complete in order, so the A chunks written here -- requested two slabs ago -- have arrived
   //         since the previous such wait).
   // ROLE 2: second K step: the B copies of the slab two ahead, into the buffer at cp_addr.
-  // EPI: the first K step of a tile -- multiplies start from zero, and the pending epilogue runs between them.
+  // EPI 1: the first K step of a tile -- multiplies start from zero, strips 4-7 of the tile before are stored between
+  //        them.  EPI 2: the last K step of a tile -- strips 0-3 are stored between its multiplies.
   auto kstep = [&](auto CURc, auto NKSc, auto MULc, auto ROLEc, uint32_t nb_off, auto EPIc, uint32_t wr_addr, auto SETc, uint32_t cp_addr) __attribute__((always_inline))  {
     constexpr int CUR = decltype(CURc)::value, NKS = decltype(NKSc)::value, ROLE = decltype(ROLEc)::value;
-    constexpr bool MUL = decltype(MULc)::value, EPI = decltype(EPIc)::value;
-    static_assert(!EPI || MUL, "the deferred epilogue rides on a multiplying K step");
+    constexpr bool MUL = decltype(MULc)::value;
+    constexpr int EPI = decltype(EPIc)::value;
+    static_assert(!EPI || MUL, "the epilogue rides on a multiplying K step");
     EpiLane e = {nullptr, nullptr, {0, 0}};
-    i32x4_t v0[2], v1[2];
-    if (EPI) {
-      e = epi_lane();
-#pragma unroll
-      for (int j = 0; j < 8; ++j) epi_cvt(e, 0, j);  // strip 0 has no multiplies in front of it to hide under
-    }
+    i32x4_t vv[2][2];
+    if (EPI && !B_KMAJOR) e = epi_lane();
+    int lane_off = 0;
+    uint2 ex = {0, 0};
+    if (EPI && B_KMAJOR) lane_off = epi_lane_t();
+    // NT: unit u = 4 (strip - first strip) + r in the gaps in front of multiplies T0 + 3 u and T0 + 3 u + 1: a strip of
+    // the tile's last K step is complete three multiplies before its first unit, a strip of the first K step is
+    // started afresh after its last unit
+    constexpr int EPI_T0 = EPI == 2 ? 11 : 0;
+    // EPI 2 (a tile's last K step) converts and stores strips 0-3 of the tile, EPI 1 (the next tile's first) strips
+    // 4-7: block bb of the half in the gap in front of multiply G0 + 7 bb / 4, at least four multiplies after the
+    // multiply that completed it and before the one that starts it afresh; a piece (four blocks) is read back in the
+    // gap of its last block and stored two and four gaps later.
+    constexpr int EPI_S0 = EPI == 2 ? 0 : 4, EPI_G0 = EPI == 2 ? 4 : 0;
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
       for (int jj = 0; jj < 8; ++jj) {
         const int j = (i & 1) ? 7 - jj : jj;  // snake order: one operand register changes per multiply
-        if (EPI) {
-          if (jj == 0) epi_read(e, 0, v0);            // strip i, staged during the previous row block
-          if (jj == 1) epi_read(e, 1, v1);
-          if (i < 7) epi_cvt(e, i + 1, jj);           // its piece's read-back has been issued (jj = 0: piece 0, jj = 4: piece 1)
-          if (jj == 3) epi_store(e, i, 0, 0, v0[0], true);
-          if (jj == 4) epi_store(e, i, 0, 1, v0[1], true);
-          if (jj == 5) epi_store(e, i, 1, 0, v1[0], true);
-          if (jj == 6) epi_store(e, i, 1, 1, v1[1], true);
-          mfma_new<DT>(acc[i][j], fb[CUR][j], fa[CUR][i]);
+        if (EPI && B_KMAJOR) {
+          const int gap = i * 8 + jj;
+#pragma unroll
+          for (int u = 0; u < 16; ++u) {
+            if (EPI_T0 + 3 * u == gap) ex = epi_half_t(EPI_S0 + u / 4, u % 4, 0);
+            if (EPI_T0 + 3 * u + 1 == gap) { const uint2 ey = epi_half_t(EPI_S0 + u / 4, u % 4, 1); epi_store_t(lane_off, EPI_S0 + u / 4, u % 4, ex, ey, true); }
+          }
+        }
+        if (EPI && !B_KMAJOR) {
+          const int gap = i * 8 + jj;
+#pragma unroll
+          for (int bb = 0; bb < 32; ++bb) {
+            const int g = EPI_G0 + 7 * bb / 4, si = EPI_S0 + bb / 8, sj = (si & 1) ? 7 - bb % 8 : bb % 8;
+            if (g == gap) epi_cvt(e, si, sj);
+            if ((bb & 3) == 3 && g == gap) epi_read(e, sj >> 2, vv[(bb >> 2) & 1]);
+          }
+#pragma unroll
+          for (int bb = 3; bb < 32; bb += 4) {
+            const int g = EPI_G0 + 7 * bb / 4, si = EPI_S0 + bb / 8, sj = (si & 1) ? 7 - bb % 8 : bb % 8;
+            if (g + 2 == gap) epi_store(e, si, sj >> 2, 0, vv[(bb >> 2) & 1][0], true);
+            if (g + 4 == gap) epi_store(e, si, sj >> 2, 1, vv[(bb >> 2) & 1][1], true);
+          }
+        }
+        if (EPI == 1) {
+          if (B_KMAJOR) mfma_new<DT>(acc[i][j], fa[CUR][i], fb[CUR][j]);
+          else mfma_new<DT>(acc[i][j], fb[CUR][j], fa[CUR][i]);
         } else if (MUL) {
-          mfma_acc<DT>(acc[i][j], fb[CUR][j], fa[CUR][i]);
+          if (B_KMAJOR) mfma_acc<DT>(acc[i][j], fa[CUR][i], fb[CUR][j]);
+          else mfma_acc<DT>(acc[i][j], fb[CUR][j], fa[CUR][i]);
         }
         const int n = i * 8 + jj;
 #define TGG_W4_RD(q) if (n == q) read_frag(std::integral_constant<int, NKS>(), std::integral_constant<int, q>(), fa[CUR ^ 1], fb[CUR ^ 1], nb_off);
@@ -423,7 +508,7 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
         }
       }
     if (ROLE == 2) asm volatile("s_waitcnt lgkmcnt(0)" : TGG_TIE8(fa[CUR ^ 1]), TGG_TIE8(fb[CUR ^ 1]) : : "memory");
-    else if (ROLE == 1) asm volatile("s_waitcnt vmcnt(%16) lgkmcnt(0)" : TGG_TIE8(fa[CUR ^ 1]), TGG_TIE8(fb[CUR ^ 1]) : "n"(EPI ? 40 : 8) : "memory");
+    else if (ROLE == 1) asm volatile("s_waitcnt vmcnt(%16) lgkmcnt(0)" : TGG_TIE8(fa[CUR ^ 1]), TGG_TIE8(fb[CUR ^ 1]) : "n"(EPI ? 24 : 8) : "memory");
     else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : TGG_TIE8(fa[CUR ^ 1]), TGG_TIE8(fb[CUR ^ 1]) : : "memory");
   };
 
@@ -455,7 +540,7 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
 #undef TGG_W4_P3
   koff_s = 3 * 128;  // at least four slabs per tile (w4_supported): both cursors are still in the first tile
   koff_d = 2 * d_step;
-  kstep(I1(), I0(), No(), I0(), 0u, No(), 0u, I0(), 0u);  // reads K step 0 of buffer 0 into set 0, multiplies nothing, waits for everything
+  kstep(I1(), I0(), No(), I0(), 0u, I0(), 0u, I0(), 0u);  // reads K step 0 of buffer 0 into set 0, multiplies nothing, waits for everything
   const int kt_all = p.K / BK4;
 
   for (int tile_id = walk.first; tile_id < walk.end; tile_id += walk.stride) {
@@ -464,30 +549,34 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
     if (!mul) epi_flush();  // no multiplies in this tile to hide the pending stores under
     // one slab; FIRST: the tile's first, whose first K step starts the accumulators afresh and carries the epilogue;
     // PAR: parity of the slab = its LDS buffer; the A chunks of the next slab wait in register set 1 - PAR
-    auto slab = [&](auto FIRST, auto PARc) __attribute__((always_inline)) {
+    auto slab = [&](auto EPc, auto PARc) __attribute__((always_inline)) {
+      typedef std::integral_constant<int, decltype(EPc)::value == 1 ? 1 : 0> Ep0;  // the tile's first slab: its first K step carries strips 4-7 of the tile before
+      typedef std::integral_constant<int, decltype(EPc)::value == 2 ? 2 : 0> Ep1;  // the tile's last slab: its second K step carries strips 0-3
       constexpr int PAR = decltype(PARc)::value;
       typedef std::integral_constant<int, 1 - PAR> SetN;
       constexpr uint32_t cur_off = PAR * C::STAGE_BYTES, nxt_off = C::STAGE_BYTES - cur_off;
-      if (mul) kstep(I0(), I1(), Yes(), I1(), cur_off, FIRST, s_wr + nxt_off, SetN(), 0u);
-      else kstep(I0(), I1(), No(), I1(), cur_off, No(), s_wr + nxt_off, SetN(), 0u);
+      if (mul) kstep(I0(), I1(), Yes(), I1(), cur_off, Ep0(), s_wr + nxt_off, SetN(), 0u);
+      else kstep(I0(), I1(), No(), I1(), cur_off, I0(), s_wr + nxt_off, SetN(), 0u);
       // set 1 is complete, this wave has read all it needs of the current slab, its copies of the next slab have landed
       asm volatile("s_barrier" ::: "memory");
-      if (mul) kstep(I1(), I0(), Yes(), I2(), nxt_off, No(), 0u, I0(), wave_buf + cur_off);
-      else kstep(I1(), I0(), No(), I2(), nxt_off, No(), 0u, I0(), wave_buf + cur_off);
+      if (mul) kstep(I1(), I0(), Yes(), I2(), nxt_off, Ep1(), 0u, I0(), wave_buf + cur_off);
+      else kstep(I1(), I0(), No(), I2(), nxt_off, I0(), 0u, I0(), wave_buf + cur_off);
     };
-    slab(Yes(), I0());  // an even number of slabs per tile: every tile starts in buffer 0
-    slab(No(), I1());
-    for (int kt = 2; kt < kt_all; kt += 2) {
-      slab(No(), I0());
-      slab(No(), I1());
+    slab(I1(), I0());  // an even number of slabs per tile, at least four: every tile starts in buffer 0
+    slab(I0(), I1());
+    for (int kt = 4; kt < kt_all; kt += 2) {
+      slab(I0(), I0());
+      slab(I0(), I1());
     }
-    // what the next tile's first K step (or the flush at the end) will store: nothing for a wave whose block of the
-    // tile has no rows or no columns
+    // what the tile's last K step, the next tile's first K step and a flush store: nothing for a wave whose block of
+    // the tile has no rows or no columns
     const int rows_left = cur.rows - wm0;
     pend_rs = make_rsrc32((uint64_t)p.C + (uint64_t)(((cur.row0 + wm0) * (int64_t)p.N + cur.n0 + wn0) * 2),
                           active ? (rows_left < 128 ? rows_left : 128) * p.N * 2 : 0);
     pend_cols = __builtin_amdgcn_readfirstlane(active ? p.N - cur.n0 - wn0 : 0);
-    pending = mul;  // a wave that sat the tile out has flushed and left nothing behind
+    pending = mul;  // a wave that sat the tile out has flushed and leaves nothing behind
+    slab(I0(), I0());
+    slab(I2(), I1());
     // both cursors are in the next tile by now: it becomes the current one, and the one after it is looked up
     cur = nxt_tile;
     const bool more = tile_at(tile_id + 2 * walk.stride, nxt_tile);
