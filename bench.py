@@ -406,12 +406,33 @@ def build_workload(name: str, dev, seed: int = 2026, zeros: bool = False, num_cu
     raise ValueError(name)
 
 
-def time_workload(fn, steps: int, warmup: int, dev):
-    """W untimed launches, then `steps` launches each bracketed by HIP events on the launch stream.
-    Returns (wall ms per step, list of per-launch event times in ms)."""
+MIN_WARM_MS = 150.0   # the clocks of a chip that has been idle settle over roughly 100 ms of work
+MIN_TIMED_MS = 60.0
+SHORT_STEP_MS = 1.5
+
+
+def time_workload(fn, steps: int, warmup: int, dev, stretch: bool = False):
+    """`warmup` untimed launches, then `steps` launches each bracketed by HIP events on the launch stream.
+    A workload whose step takes well under a millisecond would spend the whole measurement on a chip that is still
+    raising its clocks (masked decode: 0.555 ms per step after 12 warm-up launches, 0.525 after 300, same box), so the
+    warm-up of a step shorter than SHORT_STEP_MS goes on until MIN_WARM_MS of launches have been issued (steps of
+    several milliseconds measure the same either way: the requested count stands); with ``stretch`` (the secondary
+    workloads of the default line) the timed region of such a workload grows to at least MIN_TIMED_MS as well.
+    Returns (wall ms per step, list of per-launch event times in ms, launches timed, warm-up launches done)."""
+    t0 = time.perf_counter()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    done = warmup
+    step_ms = (time.perf_counter() - t0) * 1e3 / max(warmup, 1)
+    if warmup > 0 and step_ms < SHORT_STEP_MS and step_ms * warmup < MIN_WARM_MS:
+        more = min(2000, int(MIN_WARM_MS / max(step_ms, 1e-3)) + 1 - warmup)
+        for _ in range(more):
+            fn()
+        torch.cuda.synchronize()
+        done += more
+        if stretch:
+            steps = max(steps, min(2000, int(MIN_TIMED_MS / max(step_ms, 1e-3)) + 1))
     stream = torch.cuda.current_stream(dev)
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     t0 = time.perf_counter()
@@ -421,7 +442,7 @@ def time_workload(fn, steps: int, warmup: int, dev):
         e.record(stream)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return wall_ms, [s.elapsed_time(e) for s, e in evs]
+    return wall_ms, [s.elapsed_time(e) for s, e in evs], steps, done
 
 
 def summarise(name: str, flops: float, nbytes: float, dtype_tag: str, wall_ms: float, kernel_ms, default_draw: bool):
@@ -461,7 +482,7 @@ def time_vendor_dense(flops: float, steps: int, warmup: int, dev):
     vd = getattr(build_workload, "vendor_dense", None)
     if vd is None:
         return None
-    _, kms = time_workload(vd, steps, warmup, dev)
+    _, kms, _, _ = time_workload(vd, steps, warmup, dev)
     avg = sum(kms) / len(kms)
     return dict(value=round(flops / (avg * 1e-3) / 1e12, 2), unit="TFLOP/s", avg_ms=round(avg, 4), min_ms=round(min(kms), 4),
                 kind="torch.matmul (hipBLASLt): the whole A against one expert's weights, i.e. the same M x N x K as ONE dense GEMM")
@@ -698,15 +719,15 @@ def main() -> int:
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    wall_ms, kernel_ms = time_workload(fn, args.steps, args.warmup, dev)
+    wall_ms, kernel_ms, steps_done, warm_done = time_workload(fn, args.steps, args.warmup, dev)
     value, unit, roofline = summarise(workload, flops, nbytes, dtype_tag, wall_ms, kernel_ms, default_draw)
     vendor = None if args.no_vendor_loop else time_vendor_loop(flops)
     vendor_dense = None if args.no_vendor_loop else time_vendor_dense(flops, args.steps, args.warmup, dev)
     cpu_baseline = cpu_base(cpu_sample)
 
     line = {
-        "metric": METRICS[kind].replace("G=128", f"G={config['G']}") if "G" in config else METRICS[kind], "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak",
+        "metric": METRICS[kind].replace("G=128", f"G={config['G']}") if "G" in config else METRICS[kind], "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": steps_done,
+        "warmup": warm_done, "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": dtype_tag, "data": "synthetic-zeros" if args.zeros else "synthetic", "config": config,
         "roofline": roofline, "cpu_baseline": cpu_baseline, "vendor_loop": vendor,
     }
@@ -723,7 +744,7 @@ def main() -> int:
         release()
         name8 = "fp8_block_m_grouped"
         fn8, flops8, nbytes8, tag8, config8, cpu8 = build(name8)
-        wall8, kms8 = time_workload(fn8, args.steps, args.warmup, dev)
+        wall8, kms8, _, _ = time_workload(fn8, args.steps, args.warmup, dev)
         value8, unit8, roof8 = summarise(name8, flops8, nbytes8, tag8, wall8, kms8, default_draw)
         line["fp8"] = {"metric": METRICS["fp8"], "value": round(value8, 2), "unit": unit8, "ms_per_step": round(wall8, 4),
                        "dtype": tag8, "config": config8, "roofline": roof8,
@@ -735,10 +756,11 @@ def main() -> int:
                           ("quant_trans128", "quant_trans128"), ("quant_token128", "quant_token128")):
             release()
             fnx, flopsx, nbytesx, tagx, configx, _ = build(name)
-            wallx, kmsx = time_workload(fnx, args.steps, args.warmup, dev)
+            wallx, kmsx, stepsx, warmx = time_workload(fnx, args.steps, args.warmup, dev, stretch=True)
             valuex, unitx, roofx = summarise(name, flopsx, nbytesx, tagx, wallx, kmsx, default_draw)
             line[key] = {"metric": METRICS[WORKLOADS[name][0]], "value": round(valuex, 2), "unit": unitx,
-                         "ms_per_step": round(wallx, 4), "dtype": tagx, "config": configx, "roofline": roofx}
+                         "steps": stepsx, "warmup": warmx, "ms_per_step": round(wallx, 4), "dtype": tagx, "config": configx,
+                         "roofline": roofx}
             del fnx
     print(json.dumps(line))
     return 0
