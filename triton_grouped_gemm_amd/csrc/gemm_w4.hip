@@ -631,6 +631,7 @@ bool w4_supported(const GemmParams& p, int dt, int layout, bool any_size) {
   if (p.q_fmt != 0 || p.G > kFastMaxGroups) return false;
   if ((p.N & 7) != 0 || p.K < 8 || (p.K & 7) != 0) return false;
   if ((int64_t)p.K * 2 * 256 >= (1ll << 30)) return false;
+  if ((int64_t)p.N * 2 * 128 >= (1ll << 30)) return false;  // a wave's block of the output within the epilogue's 32-bit offsets, out-of-range marker included
   if (p.K % 128 != 0 || p.K < 256) return false;  // an even number of 64-deep slabs per tile, four at least
   if (any_size) return true;
   int grid = num_cus();
