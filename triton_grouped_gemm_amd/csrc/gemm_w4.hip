@@ -10,7 +10,7 @@
 // of instruction between them): a wave issues in order and a multiply keeps the matrix pipe busy for 16 cycles, so
 // one or two other instructions between two multiplies cost nothing, three or four cost 4-10 cycles of pipe time,
 // and a 16-byte-per-lane LDS write costs 13 cycles on its own (33 next to fragment reads).  Hence: never more than
-// two instructions in a gap, m0 written a multiply ahead of the copy that needs it, every per-copy address in a
+// two instructions in a gap of the slab loop proper, m0 written a multiply ahead of the copy that needs it, every per-copy address in a
 // register or an immediate, and the per-slab bookkeeping down to an offset and three selects per cursor.
 //
 // Per slab r (two LDS slab buffers, r % 2; two register sets for A chunks), per wave:
@@ -94,7 +94,7 @@ struct W4Cfg {
   static constexpr int A_BYTES = BM * BK4 * 2, B_BYTES = BN * BK4 * 2, STAGE_BYTES = A_BYTES + B_BYTES;
   static constexpr int NI_A = A_BYTES / 1024, NI_B = B_BYTES / 1024;
   static constexpr int TM = 8, TN = 8;                       // 16x16 blocks per wave: 128 x 128
-  static constexpr int EPI_PITCH = 4 * 32 + 16;              // staged piece: 16 rows x 64 outputs, row pitch in bytes
+  static constexpr int EPI_PITCH = 4 * 32 + 16;              // epilogue staging (B as [G, K, N] only); a piece: 16 rows x 64 outputs, row pitch in bytes
   static constexpr int EPI_PIECE = 16 * EPI_PITCH;
   static constexpr int EPI_WAVE_BYTES = 2 * EPI_PIECE;       // two pieces alternate
   static constexpr int SCHED_OFF = 2 * STAGE_BYTES;
@@ -420,9 +420,9 @@ __global__ __launch_bounds__(W4Cfg::THREADS) void gemm_w4_kernel(const GemmParam
   // One K step: 64 multiplies on fragment set CUR (when MUL); the 16 fragments of K step NKS of the slab at nb_off go
   // to the other set, one read after each of the first sixteen multiplies; the LDS writes and the loads and copies follow
   // behind them (reads and staged writes apart in time: 2.5 % over interleaving them through the whole K step; the
-  // loads must not slip much later, a quarter of a slab less lead costs 6 %).  At most two other instructions sit
-  // between two multiplies: a wave issues in order, and what exceeds the sixteen cycles of a multiply leaves the matrix
-  // pipe idle.
+  // loads must not slip much later, a quarter of a slab less lead costs 6 %).  Outside the two K steps that carry
+  // the epilogue at most two other instructions sit between two multiplies: a wave issues in order, and what exceeds
+  // the sixteen cycles of a multiply leaves the matrix pipe idle.
   // ROLE 0: prologue (reads only, waits for everything).
   // ROLE 1: a slab's first K step.  The A chunks of the next slab go from register set SET to LDS (wr_addr) and the
   //         chunks of the slab three ahead are requested into the same set; ends with the wait for the B copies of
