@@ -160,3 +160,62 @@ def test_four_wave_kernel_keeps_its_reserved_registers_to_itself():
     assert "gemm_w4_kernel" in text
     stray = stray_uses_of_reserved_registers(text)
     assert not stray, f"{len(stray)} compiler-generated uses of v[192:255], first: {stray[0]}"
+
+
+# The four-wave kernel's multiplies are inline assembly, so the compiler does not know when their results land: it
+# places the epilogue's v_accvgpr_read wherever the source order allows.  The source order is written so that a block
+# is read no sooner than three multiplies (48 cycles of issue) after the multiply that wrote it, or behind a
+# statement of idle cycles; this scanner checks the kept assembly for it, in text order (what crosses a loop's back
+# edge is further apart than what it sees).
+_MIN_MULTIPLIES_BETWEEN = 3
+_MIN_IDLE_WAIT_STATES = 12
+
+
+def accumulator_reads_too_early(text: str):
+    """(multiply, read, multiplies in between, idle wait states in between) for every v_accvgpr_read in a four-wave
+    kernel that follows the multiply that wrote its register too closely."""
+    bad, inside = [], False
+    last_write = {}  # accumulator register -> (index of the multiply that wrote it, its text, idle wait states issued so far)
+    n_mul, idle = 0, 0
+    for raw in text.splitlines():
+        line = raw.split(";")[0].strip()
+        if line.endswith(":") and not line.startswith("."):
+            inside = "gemm_w4_kernel" in line
+            last_write, n_mul, idle = {}, 0, 0
+            continue
+        if not inside or not line or line.startswith("."):
+            continue
+        toks = [t.strip(",") for t in line.split()]
+        if toks[0].startswith("v_mfma"):
+            for r in _regs(toks[1], "a"):
+                last_write[r] = (n_mul, line, idle)
+            n_mul += 1
+        elif toks[0] == "s_nop":
+            idle += _wait_states(line)
+        elif toks[0] == "v_accvgpr_read_b32":
+            for r in _regs(toks[2], "a"):
+                if r in last_write:
+                    at, mul, idle_then = last_write[r]
+                    between, waited = n_mul - at - 1, idle - idle_then
+                    if between < _MIN_MULTIPLIES_BETWEEN and waited < _MIN_IDLE_WAIT_STATES:
+                        bad.append((mul, line, between, waited))
+    return bad
+
+
+def test_accumulator_read_scanner_on_snippets():
+    head = "_ZN3tgg14gemm_w4_kernelILi0ELi0ELb0EEEvNS_10GemmParamsE:\n"
+    mul = lambda a: f"v_mfma_f32_16x16x32_bf16 a[{a}:{a + 3}], v[2:5], v[6:9], a[{a}:{a + 3}]\n"
+    assert len(accumulator_reads_too_early(head + mul(0) + "v_accvgpr_read_b32 v1, a2\n")) == 1
+    assert len(accumulator_reads_too_early(head + mul(0) + mul(4) + mul(8) + "v_accvgpr_read_b32 v1, a0\n")) == 1
+    assert accumulator_reads_too_early(head + mul(0) + mul(4) + mul(8) + mul(12) + "v_accvgpr_read_b32 v1, a3\n") == []
+    assert accumulator_reads_too_early(head + mul(0) + "s_nop 15\ns_nop 7\nv_accvgpr_read_b32 v1, a1\n") == []
+    assert accumulator_reads_too_early(head + mul(0) + "v_accvgpr_read_b32 v1, a9\n") == []  # another block
+    assert accumulator_reads_too_early("other_kernel:\n" + mul(0) + "v_accvgpr_read_b32 v1, a2\n") == []
+
+
+def test_four_wave_kernel_reads_no_accumulator_right_behind_its_multiply():
+    f = BUILD / "gemm_w4.gfx950.s"
+    if not f.exists():
+        pytest.skip("no device assembly in the build directory (the library was built elsewhere or not yet)")
+    found = accumulator_reads_too_early(f.read_text())
+    assert not found, f"{len(found)} reads too close behind the multiply, first: {found[0]}"
