@@ -479,10 +479,10 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
             fb[j] = load_frag(sbn + (wn0 + 16 * j) * 128);
           } else {
             if (n == C::TN * (C::TM - 2) + 1) scn = begin_slab(ring & 1, ring3);  // scalar work under a multiply
-            // block-scaled: one copy per multiply; per-channel (no folds between the multiplies, so the copies of
-            // all waves come closer together and crowd the address unit's queue): one per two multiplies, +0.9 %
-            if (BLOCK) copy_at(C::TN + n);
-            else if (n % 2 == 0) copy_at(C::TN + n / 2);
+            // one copy per two multiplies: one per multiply crowds the address unit's queue (the copies of all waves
+            // come close together) and costs 0.9 % per-channel and 1.3 % block-scaled; one per three or more delays
+            // the last copies of the slab (0.3-1.5 % slower)
+            if (n % 2 == 0) copy_at(C::TN + n / 2);
           }
           if (BLOCK && jj == 0) srow[i] *= sb_cur;
           if (BLOCK) {
