@@ -479,10 +479,12 @@ TGG_DEV void gemm_fp8_body(const GemmParams& p) {
             fb[j] = load_frag(sbn + (wn0 + 16 * j) * 128);
           } else {
             if (n == C::TN * (C::TM - 2) + 1) scn = begin_slab(ring & 1, ring3);  // scalar work under a multiply
-            // one copy per two multiplies: one per multiply crowds the address unit's queue (the copies of all waves
-            // come close together) and costs 0.9 % per-channel and 1.3 % block-scaled; one per three or more delays
-            // the last copies of the slab (0.3-1.5 % slower)
-            if (n % 2 == 0) copy_at(C::TN + n / 2);
+            // block-scaled: one copy per two multiplies.  One per multiply crowds the address unit's queue (the copies
+            // of all waves come close together: 1.3 % slower), one per three or more delays the slab's last copies
+            // (0.3-1.5 % slower).  Per-channel, with no folds between the multiplies, the copies come closer still: one
+            // per four multiplies (1 % over one per two, 2 % over one per multiply; one per six is back at one per two)
+            if (BLOCK) { if (n % 2 == 0) copy_at(C::TN + n / 2); }
+            else if (n % 4 == 0) copy_at(C::TN + n / 4);
           }
           if (BLOCK && jj == 0) srow[i] *= sb_cur;
           if (BLOCK) {
